@@ -1,6 +1,6 @@
 """Build libqserve_amd.so (hand-written HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
-    python -m qserve_amd.build [--force] [--debug-asm]
+    python -m qserve_amd.build [--force]
 
 hipcc cross-compiles without a GPU, so this runs in the authoring container as well as on the MI355X box.
 The .so lands in qserve_amd/ (git-ignored, but shipped to the GPU box by gpurun).
@@ -77,11 +77,7 @@ def build(force=False, verbose=True, extra=(), timing=False):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
-    ap.add_argument("--debug-asm", action="store_true",
-                    help="keep the gfx950 assembly of every kernel next to the objects (qserve_amd/_build/*.s) and print "
-                         "the per-kernel register / LDS / scratch usage (implies --force)")
     ap.add_argument("--timing", action="store_true", help="build libqserve_amd_timing.so (-DQS_TIMING) instead")
     a = ap.parse_args()
-    extra = ["-save-temps=obj", "-Rpass-analysis=kernel-resource-usage"] if a.debug_asm else []
-    build(force=a.force or a.debug_asm, extra=extra, timing=a.timing)
+    build(force=a.force, timing=a.timing)
     sys.exit(0)

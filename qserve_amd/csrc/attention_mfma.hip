@@ -477,7 +477,7 @@ __global__ __launch_bounds__(NWT * 64, 4) void decode_attention_mfma_kernel(
     float m_run = -3.0e38f, l_part = 0.f, corr = 0.f, psum = 0.f;   // psum = sum of P' (removes the V operand offsets)
 
     // Lane-constant LDS addresses and the Q.K^T B operand stay in registers across the unit loop (the unit form of the
-    // loop needs ~30 registers fewer than the page form did, so nothing spills: tests/test_kernel_contracts.py)
+    // loop needs ~30 registers fewer than the page form did, so nothing spills)
     constexpr int NS = GP == 4 ? 2 : 4;     // scores per lane in the compacted softmax
     // this lane's tokens there: 16 t + 4 tg + r0 + {0 .. NS-1}
     //   GP = 4: lane li = h + 4 (2 t + rp): r0 = 2 rp;   GP = 8: lane li = h + 8 t: r0 = 0

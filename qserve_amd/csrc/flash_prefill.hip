@@ -201,8 +201,8 @@ __global__ __launch_bounds__(64 * NWV, QS_FLASH_OCC) void flash_fwd_kernel(const
     // (s_waitcnt vmcnt(7) ... vmcnt(0), one per fragment).  The hardware counter it waits on also counts the LDS-DMA of tile
     // t + 1, issued a few instructions earlier by asm the compiler does not see either: every wave sat through the L2 round trip
     // of its own prefetch inside Q.K^T of every tile (the "1 430 cycles for DMA issue + Q.K^T" of the round-2 trace, 512 of them
-    // MFMA).  An empty asm that rewrites the fragments makes the compiler wait HERE, once (tests/test_kernel_contracts.py pins:
-    // no vmcnt wait between the loop's barriers other than the explicit one of tiles_landed()).
+    // MFMA).  An empty asm that rewrites the fragments makes the compiler wait HERE, once, so that
+    // the only vmcnt wait between the loop's barriers is the explicit one of tiles_landed().
     if constexpr (R6) {
 #pragma unroll
         for (int s = 0; s < 8; ++s) asm volatile("" : "+v"(qf[s]));

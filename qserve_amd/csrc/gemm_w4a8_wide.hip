@@ -73,9 +73,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // acc(mt, cl) = a[(4 mt + cl) 4 .. + 3].  FIRST: the tile's first stage writes A x B + 0 (no zero-fill of 256 registers).
-// No hazard padding is needed inside: the operands are LDS read results or were built a whole stage earlier (the disassembly
-// contract in tests/test_kernel_contracts.py checks that no VALU write of a source precedes an MFMA by fewer than two
-// instructions), and an accumulate chain on the same registers needs no wait states.
+// No hazard padding is needed inside: the operands are LDS read results or were built a whole stage earlier, and an accumulate chain on the same registers needs no wait states.
 template <int ACC, bool FIRST>
 __device__ __forceinline__ void mfma_acc(const v4i& a, const v4i& b) {
     if constexpr (FIRST)

@@ -1,5 +1,5 @@
 // Round 5: is ONE wave per SIMD able to keep the INT8 matrix pipe busy?  scripts/microbench_mfma3.hip (round 2) said no - 2.09 POPS
-// for a 128 x 128 wave tile - and the 4-wave / 512-register tile was dropped on that number.  Its ISA (hipcc -save-temps) shows why:
+// for a 128 x 128 wave tile - and the 4-wave / 512-register tile was dropped on that number.  The reason:
 // with 256 accumulator registers the register allocator fails to coalesce the loop-carried accumulator tuples and rotates half of
 // them through v_accvgpr_mov copies (212 copies + 108 s_nop per 64 MFMAs).  The measurement was of the compiler, not of the SIMD.
 // Here the MFMAs are inline asm on FIXED accumulator registers a[0:255] (nothing for the allocator to decide):
