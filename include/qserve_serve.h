@@ -1,0 +1,76 @@
+/* qserve_serve.h -- C ABI of libqserve_serve.so: the kernels of the paged serving engine (qserve_amd/serving).
+ *
+ * Every tensor is a device pointer; `dtype` selects the storage type of activations, weights and cache rows
+ * (QSV_BF16 = bfloat16 with 32-bit accumulation, QSV_F32 = float everywhere).  The residual stream, norm statistics,
+ * attention scores / weights, rotary angles and router scores are float in both modes.  All launches go to `stream`
+ * (a hipStream_t) and return 0 or an error code; qsv_last_error() describes the last failure of the calling thread.
+ */
+#pragma once
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QSV_OK 0
+#define QSV_EINVAL 1
+#define QSV_BF16 0
+#define QSV_F32 1
+
+int qsv_version(void);
+const char* qsv_arch(void);
+const char* qsv_last_error(void);
+
+/* x[t] = table[tokens[t]] (float) and h[t] = the same row in the storage type. */
+int qsv_embed(float* x, void* h, const void* table, const int32_t* tokens, int n_tokens, int width, int dtype, void* stream);
+
+/* x[t] += layer_norm(y[t]) * w (no bias; variance = mean of squared deviations); h[t] = x[t] in the storage type. */
+int qsv_add_layer_norm(float* x, void* h, const void* y, const void* w, float eps, int n_tokens, int width, int dtype,
+                       void* stream);
+
+/* out[r] = layer_norm(x[rows[r]]) * w in the storage type (rows == NULL: row r). */
+int qsv_layer_norm_rows(void* out, const float* x, const int32_t* rows, const void* w, float eps, int n_rows, int width,
+                        int dtype, void* stream);
+
+/* Latent projections of one attention layer, per token t, from `down` (row stride down_stride elements):
+ *   cq[t]            = rms_norm(down[t, q_off : q_off + q_rank]) * q_w
+ *   pool[slot[t]]    = [ rms_norm(down[t, kv_off : kv_off + kv_rank]) * kv_w | rot(down[t, kv_off + kv_rank : + rot_dim]) ]
+ * rot() rotates the pairs (2i, 2i+1), i < rot_n / 2, by the angle whose cos / sin are rope[pos[t]][0 / 1][i]
+ * (rope: float [positions, 2, rot_n / 2], already scaled); the remaining rot_dim - rot_n values are copied.
+ * Cache rows have row_width = kv_rank + rot_dim elements. */
+int qsv_latent_prep(const void* down, int64_t down_stride, int q_off, int q_rank, const void* q_w, void* cq,
+                    int kv_off, int kv_rank, const void* kv_w, int rot_dim, int rot_n, const float* rope,
+                    void* pool, const int64_t* slot, const int32_t* pos, float eps, int n_tokens, int dtype, void* stream);
+
+/* qf[t, h] = scale * [ q_abs[h, t, 0 : rank] | rot(q[t, h, dim : dim + rot_dim]) ]  (float [T, H, rank + rot_dim]).
+ * q: [T, H, dim + rot_dim], q_abs: [H, T, rank] (the query carried into the latent space), both in the storage type. */
+int qsv_latent_query(float* qf, const void* q, const void* q_abs, const float* rope, const int32_t* pos, float scale,
+                     int n_tokens, int heads, int dim, int rot_dim, int rot_n, int rank, int dtype, void* stream);
+
+/* Softmax attention of every token over the cached latent rows of its sequence:
+ *   score(t, h, j) = qf[t, h] . pool[row(seq[t], j)]   for  max(0, pos[t] - window + 1) <= j <= pos[t]  (window 0: all j <= pos)
+ *   out[t, h]      = sum_j softmax_j(score) * pool[row][0 : rank]            (storage type, [T, H, rank])
+ * row(s, j) = block_table[s * table_stride + j / page] * page + j % page.  variant: 0 = default kernel choice. */
+int qsv_latent_attention(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
+                         const int32_t* seq, const int32_t* pos, int window, int n_tokens, int heads, int rank,
+                         int row_width, int page, int dtype, int variant, void* stream);
+
+/* o[t, i] *= sigmoid(g[t * g_stride + i]),  i < n. */
+int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int n, int dtype, void* stream);
+
+/* Grouped top-k router: scores = softmax(router . h[t]) over n_experts; the experts form n_groups equal groups of neighbours,
+ * a group's score is its largest score, only experts of the best keep_groups groups are eligible; the top_k eligible experts
+ * with the largest scores are chosen.  idx [T, top_k] int32, weight [T, top_k] float = their scores (not renormalised). */
+int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, int n_tokens, int width, int n_experts,
+                  int top_k, int n_groups, int keep_groups, int dtype, void* stream);
+
+/* act[t, k] = relu(up[idx[t, k]] . h[t])^2     up: [E, ff, width] -> act [T, top_k, ff] (storage type). */
+int qsv_moe_up(void* act, const void* h, const void* up, const int32_t* idx, int n_tokens, int top_k, int width, int ff,
+               int dtype, void* stream);
+
+/* y[t] = sum_k weight[t, k] * down[idx[t, k]] . act[t, k]     down: [E, width, ff] -> y [T, width] (storage type). */
+int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx, const float* weight, int n_tokens,
+                 int top_k, int width, int ff, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -74,10 +74,65 @@ def build(force=False, verbose=True, extra=(), timing=False):
     return lib
 
 
+# ---- libqserve_serve.so: the kernels of the paged serving engine (qserve_amd/serving) -------------------------------------------
+# A library of its own: a model served by that engine needs these few translation units only, so its first start in a fresh
+# checkout compiles them (a minute) and not the W4A8 GEMM / KV4 attention families above.
+SERVE_CSRC = os.path.join(CSRC, "serve")
+SERVE_BUILD = os.path.join(HERE, "_build_serve")
+SERVE_LIB = os.path.join(HERE, "libqserve_serve.so")
+SERVE_SOURCES = ["serve_rows.hip", "serve_attention.hip", "serve_moe.hip"]
+# packed-FP32 instructions off: the kernels' float statistics must not depend on how the compiler pairs them
+SERVE_FLAGS = FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def serve_stale():
+    """True if libqserve_serve.so is missing or older than one of its sources."""
+    if not os.path.exists(SERVE_LIB):
+        return True
+    deps = [os.path.join(SERVE_CSRC, f) for f in os.listdir(SERVE_CSRC)]
+    deps.append(os.path.join(os.path.dirname(HERE), "include", "qserve_serve.h"))
+    return os.path.getmtime(SERVE_LIB) < max(os.path.getmtime(d) for d in deps)
+
+
+def build_serve(force=False, verbose=True):
+    os.makedirs(SERVE_BUILD, exist_ok=True)
+    hdr = max(os.path.getmtime(os.path.join(SERVE_CSRC, f)) for f in os.listdir(SERVE_CSRC) if f.endswith(".h"))
+    hdr = max(hdr, os.path.getmtime(os.path.join(os.path.dirname(HERE), "include", "qserve_serve.h")))
+
+    def one(src):
+        srcp, obj = os.path.join(SERVE_CSRC, src), os.path.join(SERVE_BUILD, src.replace(".hip", ".o"))
+        if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(srcp), hdr):
+            return obj, False
+        r = subprocess.run([hipcc(), *SERVE_FLAGS, "-c", srcp, "-o", obj], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr[-4000:]}")
+        return obj, True
+
+    with cf.ThreadPoolExecutor(max_workers=min(8, len(SERVE_SOURCES))) as ex:
+        res = list(ex.map(one, SERVE_SOURCES))
+    if force or any(r for _, r in res) or not os.path.exists(SERVE_LIB):
+        tmp = SERVE_LIB + f".tmp{os.getpid()}"           # (renamed into place: a process loading the library never sees half of it)
+        r = subprocess.run([hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wl,--no-undefined", *[o for o, _ in res],
+                            "-o", tmp], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+        os.replace(tmp, SERVE_LIB)
+        if verbose:
+            print(f"[qserve_amd.build] linked {SERVE_LIB}", file=sys.stderr)
+    elif verbose:
+        print(f"[qserve_amd.build] up to date: {SERVE_LIB}", file=sys.stderr)
+    return SERVE_LIB
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--serve", action="store_true", help="build only libqserve_serve.so (the paged serving engine's kernels)")
     ap.add_argument("--timing", action="store_true", help="build libqserve_amd_timing.so (-DQS_TIMING) instead")
     a = ap.parse_args()
+    if a.serve:
+        build_serve(force=a.force)
+        sys.exit(0)
     build(force=a.force, timing=a.timing)
+    build_serve(force=a.force)
     sys.exit(0)

@@ -1,0 +1,139 @@
+// serve_attention.hip -- softmax attention over a paged cache of latent rows (one row per token, shared by all heads).
+//
+// The query arrives already carried into the latent space (qsv_latent_query), so a score is one dot product of the query
+// with a cache row and the output is the softmax-weighted sum of the rows' first `rank` elements.  One launch serves
+// prompt portions and single decoded tokens alike: every token brings its own sequence, position and window start.
+//
+// Wave kernel: workgroup = one (token, head), four waves; wave w takes keys lo + KG (w + 4 n) ... in groups of KG, lanes
+// spread over the row's elements (coalesced row reads), one butterfly reduction per score, online softmax per group, the
+// four partial results merged through LDS.  Scores, weights and sums are float.
+#include "serve_common.h"
+
+namespace {
+constexpr int NW = 4;    // waves per workgroup
+constexpr int KG = 4;    // keys per softmax update
+
+template <typename T, int EPL>
+__global__ __launch_bounds__(64 * NW) void latent_attention_wave_kernel(
+    T* __restrict__ out, const float* __restrict__ qf, const T* __restrict__ pool, const int32_t* __restrict__ block_table,
+    int table_stride, const int32_t* __restrict__ seq, const int32_t* __restrict__ pos, int window, int H, int rank, int R,
+    int page) {
+    __shared__ float s_m[NW], s_l[NW];
+    __shared__ float s_acc[NW][64 * EPL];
+    const size_t t = blockIdx.x / H;
+    const int h = blockIdx.x % H;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int p = pos[t];
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int32_t* bt = block_table + (size_t)seq[t] * table_stride;
+    const float* qrow = qf + (t * H + h) * (size_t)R;
+    float q[EPL], acc[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        q[i] = e < R ? qrow[e] : 0.f;
+        acc[i] = 0.f;
+    }
+    float m = -INFINITY, l = 0.f;
+    for (int j0 = lo + w * KG; j0 <= p; j0 += NW * KG) {
+        float c[KG][EPL], s[KG];
+#pragma unroll
+        for (int k = 0; k < KG; ++k) {
+            const int j = j0 + k;
+            const bool ok = j <= p;
+            const int jj = ok ? j : p;
+            const T* row = pool + ((size_t)bt[jj / page] * page + (size_t)(jj % page)) * (size_t)R;
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) {
+                const int e = lane + 64 * i;
+                c[k][i] = e < R ? ld(row, e) : 0.f;
+                d += q[i] * c[k][i];
+            }
+            d = wave_sum(d);
+            s[k] = ok ? d : -INFINITY;
+        }
+        float mx = m;
+#pragma unroll
+        for (int k = 0; k < KG; ++k) mx = fmaxf(mx, s[k]);
+        const float alpha = expf(m - mx);          // first group: exp(-inf) = 0 (mx is finite: key j0 is visible)
+        float pk[KG], ps = 0.f;
+#pragma unroll
+        for (int k = 0; k < KG; ++k) {
+            pk[k] = expf(s[k] - mx);
+            ps += pk[k];
+        }
+        l = l * alpha + ps;
+        m = mx;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            float a = acc[i] * alpha;
+#pragma unroll
+            for (int k = 0; k < KG; ++k) a += pk[k] * c[k][i];
+            acc[i] = a;
+        }
+    }
+    if (lane == 0) {
+        s_m[w] = m;
+        s_l[w] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) s_acc[w][lane + 64 * i] = acc[i];
+    __syncthreads();
+    float M = s_m[0];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) M = fmaxf(M, s_m[k]);
+    float f[NW], L = 0.f;
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+        f[k] = expf(s_m[k] - M);                   // a wave without keys has m = -inf: factor 0
+        L += f[k] * s_l[k];
+    }
+    const float invL = 1.0f / L;
+    T* o = out + (t * H + h) * (size_t)rank;
+    for (int e = threadIdx.x; e < rank; e += 64 * NW) {
+        float a = 0.f;
+#pragma unroll
+        for (int k = 0; k < NW; ++k) a += f[k] * s_acc[k][e];
+        st(o, e, a * invL);
+    }
+}
+
+template <typename T>
+int launch_wave(void* out, const float* qf, const void* pool, const int32_t* bt, int ts, const int32_t* seq, const int32_t* pos,
+                int window, int n, int H, int rank, int R, int page, hipStream_t st_) {
+    const dim3 grid(n * H), block(64 * NW);
+#define QSV_ATT(E)                                                                                                        \
+    hipLaunchKernelGGL((latent_attention_wave_kernel<T, E>), grid, block, 0, st_, (T*)out, qf, (const T*)pool, bt, ts, seq, pos, \
+                       window, H, rank, R, page)
+    if (R <= 64) QSV_ATT(1);
+    else if (R <= 128) QSV_ATT(2);
+    else if (R <= 192) QSV_ATT(3);
+    else if (R <= 256) QSV_ATT(4);
+    else if (R <= 384) QSV_ATT(6);
+    else if (R <= 576) QSV_ATT(9);
+    else {
+        qsv_set_error("qsv_latent_attention: cache rows of %d elements (at most 576)", R);
+        return QSV_EINVAL;
+    }
+#undef QSV_ATT
+    return QSV_OK;
+}
+}  // namespace
+
+extern "C" int qsv_latent_attention(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
+                                    const int32_t* seq, const int32_t* pos, int window, int n, int H, int rank, int R, int page,
+                                    int dtype, int variant, void* stream) {
+    QSV_REQUIRE(out && qf && pool && block_table && seq && pos, "qsv_latent_attention: null argument");
+    QSV_REQUIRE(n >= 0 && H > 0 && rank > 0 && R >= rank && page > 0 && table_stride > 0 && window >= 0,
+                "qsv_latent_attention: bad sizes");
+    if (n == 0) return QSV_OK;
+    QSV_REQUIRE((int64_t)n * H < (1ll << 31), "qsv_latent_attention: too many (token, head) pairs");
+    (void)variant;
+    int rc = QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_latent_attention",
+                 rc = launch_wave<T>(out, qf, pool, block_table, table_stride, seq, pos, window, n, H, rank, R, page,
+                                     (hipStream_t)stream));
+    if (rc != QSV_OK) return rc;
+    return qsv_launch_status("qsv_latent_attention");
+}

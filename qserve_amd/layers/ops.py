@@ -1,0 +1,239 @@
+"""The operations the served models are made of, in two forms with one signature:
+
+* `HipOps`   - the product path: one launch of libqserve_serve.so per call (include/qserve_serve.h), on the current stream;
+* `TorchOps` - the same operations written with unfused torch tensor ops on any device.  It exists to bring a layer up and
+  to test host logic (cache, scheduler, batching) where no GPU is; an engine only uses it when asked to by name - a model on
+  a GPU never falls back to it.
+
+Conventions: `x` is the float residual stream [T, D]; `h` and every other activation is in the storage type (bfloat16 or
+float32); matrix products are the vendor's (`linear`), with float accumulation.
+"""
+import torch
+
+BF16, F32 = 0, 1
+
+
+def dtype_code(dtype):
+    if dtype == torch.bfloat16:
+        return BF16
+    if dtype == torch.float32:
+        return F32
+    raise ValueError(f"the serving kernels store bfloat16 or float32, not {dtype}")
+
+
+def linear(x, w):
+    """x [T, in] @ w [out, in]^T in the storage type (hipBLASLt / rocBLAS through torch; float accumulation)."""
+    return torch.matmul(x, w.t())
+
+
+class HipOps:
+    name = "hip"
+
+    def __init__(self, dtype):
+        from ..serving._lib import check, lib
+        self.dtype, self.code = dtype, dtype_code(dtype)
+        self.L, self.check = lib(), check
+
+    @staticmethod
+    def _s():
+        return torch.cuda.current_stream().cuda_stream
+
+    def _need(self, *ts):
+        for t in ts:
+            if t is not None and not (t.is_cuda and t.is_contiguous()):
+                raise RuntimeError("serving kernels need contiguous tensors on the GPU")
+
+    def embed(self, tokens, table):
+        T, D = tokens.numel(), table.size(1)
+        x = torch.empty((T, D), dtype=torch.float32, device=table.device)
+        h = torch.empty((T, D), dtype=self.dtype, device=table.device)
+        self._need(tokens, table)
+        self.check(self.L.qsv_embed(x.data_ptr(), h.data_ptr(), table.data_ptr(), tokens.data_ptr(), T, D, self.code, self._s()),
+                   "embed")
+        return x, h
+
+    def add_layer_norm(self, x, y, w, eps):
+        """x += layer_norm(y) * w in place; returns x in the storage type."""
+        h = torch.empty(x.shape, dtype=self.dtype, device=x.device)
+        self._need(x, y, w)
+        assert y.shape == x.shape and y.dtype == self.dtype and x.dtype == torch.float32
+        self.check(self.L.qsv_add_layer_norm(x.data_ptr(), h.data_ptr(), y.data_ptr(), w.data_ptr(), eps, x.size(0), x.size(1),
+                                             self.code, self._s()), "add_layer_norm")
+        return h
+
+    def layer_norm_rows(self, x, rows, w, eps):
+        n = x.size(0) if rows is None else rows.numel()
+        out = torch.empty((n, x.size(1)), dtype=self.dtype, device=x.device)
+        self._need(x, rows, w)
+        self.check(self.L.qsv_layer_norm_rows(out.data_ptr(), x.data_ptr(), 0 if rows is None else rows.data_ptr(), w.data_ptr(),
+                                              eps, n, x.size(1), self.code, self._s()), "layer_norm_rows")
+        return out
+
+    def latent_prep(self, down, q_off, q_rank, q_w, kv_off, kv_rank, kv_w, rot_dim, rot_n, rope, pool, slot, pos, eps):
+        T = down.size(0)
+        cq = torch.empty((T, q_rank), dtype=self.dtype, device=down.device)
+        self._need(down, q_w, kv_w, rope, pool, slot, pos)
+        assert pool.size(-1) == kv_rank + rot_dim and slot.dtype == torch.int64 and pos.dtype == torch.int32
+        assert rope is None or (rope.dtype == torch.float32 and rope.size(-1) * 2 == rot_n)
+        self.check(self.L.qsv_latent_prep(down.data_ptr(), down.stride(0), q_off, q_rank, q_w.data_ptr(), cq.data_ptr(), kv_off,
+                                          kv_rank, kv_w.data_ptr(), rot_dim, rot_n, 0 if rope is None else rope.data_ptr(),
+                                          pool.data_ptr(), slot.data_ptr(), pos.data_ptr(), eps, T, self.code, self._s()),
+                   "latent_prep")
+        return cq
+
+    def latent_query(self, q, q_abs, rope, pos, scale, heads, dim, rot_dim, rot_n, rank):
+        T = q.size(0)
+        qf = torch.empty((T, heads, rank + rot_dim), dtype=torch.float32, device=q.device)
+        self._need(q, q_abs, rope, pos)
+        assert q.numel() == T * heads * (dim + rot_dim) and q_abs.shape == (heads, T, rank)
+        self.check(self.L.qsv_latent_query(qf.data_ptr(), q.data_ptr(), q_abs.data_ptr(), 0 if rope is None else rope.data_ptr(),
+                                           pos.data_ptr(), scale, T, heads, dim, rot_dim, rot_n, rank, self.code, self._s()),
+                   "latent_query")
+        return qf
+
+    def latent_attention(self, qf, pool, block_table, seq, pos, window, rank, page, variant=0):
+        T, H, R = qf.shape
+        out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
+        self._need(qf, pool, block_table, seq, pos)
+        assert pool.size(-1) == R and block_table.dtype == torch.int32 and seq.dtype == torch.int32
+        self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
+                                               block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
+                                               rank, R, page, self.code, variant, self._s()), "latent_attention")
+        return out
+
+    def sigmoid_gate(self, o, g):
+        """o [T, n] *= sigmoid(g [T, n]) in place; g may be a column slice of a wider matrix."""
+        self._need(o)
+        assert g.is_cuda and g.stride(1) == 1 and g.shape == o.shape
+        self.check(self.L.qsv_sigmoid_gate(o.data_ptr(), g.data_ptr(), g.stride(0), o.size(0), o.size(1), self.code, self._s()),
+                   "sigmoid_gate")
+        return o
+
+    def moe_route(self, h, router, top_k, groups, keep):
+        T, E = h.size(0), router.size(0)
+        idx = torch.empty((T, top_k), dtype=torch.int32, device=h.device)
+        wt = torch.empty((T, top_k), dtype=torch.float32, device=h.device)
+        self._need(h, router)
+        self.check(self.L.qsv_moe_route(idx.data_ptr(), wt.data_ptr(), h.data_ptr(), router.data_ptr(), T, h.size(1), E, top_k,
+                                        groups, keep, self.code, self._s()), "moe_route")
+        return idx, wt
+
+    def moe_experts(self, h, up, down, idx, wt):
+        """up [E, ff, D], down [E, D, ff]; y[t] = sum_k wt[t, k] * down[idx[t, k]] relu(up[idx[t, k]] h[t])^2."""
+        T, D = h.shape
+        top_k, ff = idx.size(1), up.size(1)
+        act = torch.empty((T, top_k, ff), dtype=self.dtype, device=h.device)
+        y = torch.empty((T, D), dtype=self.dtype, device=h.device)
+        self._need(h, up, down, idx, wt)
+        assert up.shape[2] == D and down.shape == (up.size(0), D, ff)
+        self.check(self.L.qsv_moe_up(act.data_ptr(), h.data_ptr(), up.data_ptr(), idx.data_ptr(), T, top_k, D, ff, self.code,
+                                     self._s()), "moe_up")
+        self.check(self.L.qsv_moe_down(y.data_ptr(), act.data_ptr(), down.data_ptr(), idx.data_ptr(), wt.data_ptr(), T, top_k, D,
+                                       ff, self.code, self._s()), "moe_down")
+        return y
+
+
+def _rotate(v, rope, pos, rot_n):
+    """Interleaved-pair rotation of the first rot_n columns of v [..., n] (float); rope [P, 2, rot_n / 2]."""
+    if not rot_n:
+        return v
+    cs = rope[pos.long()]                       # [T, 2, half]
+    c, s = cs[:, 0], cs[:, 1]
+    while c.dim() < v.dim():
+        c, s = c.unsqueeze(1), s.unsqueeze(1)
+    a, b = v[..., 0:rot_n:2], v[..., 1:rot_n:2]
+    out = v.clone()
+    out[..., 0:rot_n:2] = a * c - b * s
+    out[..., 1:rot_n:2] = b * c + a * s
+    return out
+
+
+class TorchOps:
+    """Unfused tensor-op form of HipOps (see the module docstring).  Same storage roundings at the same places."""
+    name = "unfused"
+
+    def __init__(self, dtype):
+        self.dtype = dtype
+        dtype_code(dtype)
+
+    def embed(self, tokens, table):
+        h = table[tokens.long()]
+        return h.float(), h.to(self.dtype)
+
+    @staticmethod
+    def _ln(y, w, eps):
+        y = y.float()
+        mu = y.mean(-1, keepdim=True)
+        var = ((y - mu) ** 2).mean(-1, keepdim=True)
+        return (y - mu) / torch.sqrt(var + eps) * w.float()
+
+    def add_layer_norm(self, x, y, w, eps):
+        x += self._ln(y, w, eps)
+        return x.to(self.dtype)
+
+    def layer_norm_rows(self, x, rows, w, eps):
+        return self._ln(x if rows is None else x[rows.long()], w, eps).to(self.dtype)
+
+    @staticmethod
+    def _rms(v, w, eps):
+        v = v.float()
+        return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * w.float()
+
+    def latent_prep(self, down, q_off, q_rank, q_w, kv_off, kv_rank, kv_w, rot_dim, rot_n, rope, pool, slot, pos, eps):
+        cq = self._rms(down[:, q_off:q_off + q_rank], q_w, eps).to(self.dtype)
+        c = self._rms(down[:, kv_off:kv_off + kv_rank], kv_w, eps)
+        kr = _rotate(down[:, kv_off + kv_rank:kv_off + kv_rank + rot_dim].float(), rope, pos, rot_n)
+        pool[slot] = torch.cat([c, kr], dim=-1).to(self.dtype)
+        return cq
+
+    def latent_query(self, q, q_abs, rope, pos, scale, heads, dim, rot_dim, rot_n, rank):
+        T = q.size(0)
+        qr = _rotate(q.view(T, heads, dim + rot_dim)[..., dim:].float(), rope, pos, rot_n)
+        return (torch.cat([q_abs.transpose(0, 1).float(), qr], dim=-1) * scale).contiguous()
+
+    def latent_attention(self, qf, pool, block_table, seq, pos, window, rank, page, variant=0):
+        T, H, R = qf.shape
+        out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
+        bt = block_table.long()
+        for t in range(T):
+            p = int(pos[t])
+            lo = max(0, p - window + 1) if window else 0
+            j = torch.arange(lo, p + 1, device=qf.device)
+            rows = pool[bt[int(seq[t]), j // page] * page + j % page].float()        # [n, R]
+            w = torch.softmax(qf[t] @ rows.t(), dim=-1)                              # [H, n]
+            out[t] = (w @ rows[:, :rank]).to(self.dtype)
+        return out
+
+    def sigmoid_gate(self, o, g):
+        o.copy_((o.float() * torch.sigmoid(g.float())).to(self.dtype))
+        return o
+
+    def moe_route(self, h, router, top_k, groups, keep):
+        s = torch.softmax(h.float() @ router.float().t(), dim=-1)
+        T, E = s.shape
+        gs = s.view(T, groups, E // groups).amax(-1)
+        kept = torch.zeros_like(gs, dtype=torch.bool).scatter_(1, gs.topk(keep, dim=-1).indices, True)
+        ok = kept[:, :, None].expand(T, groups, E // groups).reshape(T, E)
+        idx = s.masked_fill(~ok, -1.0).topk(top_k, dim=-1).indices
+        return idx.int(), s.gather(1, idx)
+
+    def moe_experts(self, h, up, down, idx, wt):
+        T, D = h.shape
+        y = torch.zeros((T, D), dtype=torch.float32, device=h.device)
+        for k in range(idx.size(1)):
+            e = idx[:, k].long()
+            a = torch.relu(torch.einsum("tfd,td->tf", up[e].float(), h.float())) ** 2
+            a = a.to(self.dtype).float()
+            y += wt[:, k, None] * torch.einsum("tdf,tf->td", down[e].float(), a)
+        return y.to(self.dtype)
+
+
+def make_ops(backend, dtype, device):
+    """backend: "hip" (the only one a served model uses) or "unfused" (bring-up and host-logic tests)."""
+    if backend == "hip":
+        if torch.device(device).type != "cuda":
+            raise RuntimeError("the hip backend needs a GPU device; there is no CPU path for served models")
+        return HipOps(dtype)
+    if backend == "unfused":
+        return TorchOps(dtype)
+    raise ValueError(f"unknown backend {backend!r}")

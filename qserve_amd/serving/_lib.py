@@ -1,0 +1,52 @@
+"""ctypes binding of libqserve_serve.so (include/qserve_serve.h): the kernels of the paged serving engine.
+
+The library is loaded on first use.  If it has not been built yet it is built then (hipcc, a few seconds); a build or load
+failure raises - on a GPU there is no other compute path.
+"""
+import ctypes as C
+import os
+import threading
+
+_vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float
+SIGNATURES = {
+    "qsv_version": (_i, []),
+    "qsv_arch": (C.c_char_p, []),
+    "qsv_last_error": (C.c_char_p, []),
+    "qsv_embed": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "qsv_add_layer_norm": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _vp]),
+    "qsv_layer_norm_rows": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _vp]),
+    "qsv_latent_prep": (_i, [_vp, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _i, _vp]),
+    "qsv_latent_query": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "qsv_latent_attention": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "qsv_sigmoid_gate": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp]),
+    "qsv_moe_route": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "qsv_moe_up": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "qsv_moe_down": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            from .. import build as b
+            path = os.environ.get("QS_SERVE_LIBRARY") or b.SERVE_LIB
+            if not os.path.exists(path):
+                b.build_serve(verbose=True)
+            L = C.CDLL(path)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(L, name)              # AttributeError if the built library is older than this binding: loud by design
+                fn.restype, fn.argtypes = res, args
+            _lib = L
+    return _lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = lib().qsv_last_error()
+        raise RuntimeError(f"{what}: {msg.decode() if msg else 'error'} (code {rc})")

@@ -1,0 +1,140 @@
+"""The serving engine: a registered model + the paged cache + the scheduler + the sampler.
+
+`Engine.step()` is the generation path: schedule -> `execute` -> sample -> book-keeping.  `execute` is the step function -
+it lays the scheduled tokens out as one flat batch (token, sequence slot, position, cache row per token), runs the model
+over it and returns float logits at the rows asked for.  Callers that bring their own tokens (a recorded trace, a test)
+use `open_sequence` / `execute` / `close_sequence` directly and so drive the very same cache and kernels.
+"""
+import itertools
+from dataclasses import dataclass
+
+import torch
+
+from ..layers.ops import make_ops
+from . import registry
+from .cache import PagedCache
+from .sampler import SamplingParams, sample
+from .scheduler import Request, Scheduler
+
+DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclass
+class StepBatch:
+    """One step's tokens as the kernels read them (device tensors unless noted)."""
+    tokens: torch.Tensor        # int32 [T]
+    seq: torch.Tensor           # int32 [T]  sequence slot (row of the block table)
+    pos: torch.Tensor           # int32 [T]  position in its sequence
+    slot: torch.Tensor          # int64 [T]  flat cache row the token's state is written to
+    block_table: torch.Tensor   # int32 [slots, pages]
+    max_pos: int                # host: largest position in the batch
+    n_tokens: int
+
+
+class Engine:
+    def __init__(self, model_cls, config, weights, dtype="bfloat16", device="cuda:0", max_tokens=4096, max_seqs=4,
+                 backend="hip", max_batch_tokens=2048, prefill_chunk=512, page=64):
+        self.dtype = DTYPES[dtype] if isinstance(dtype, str) else dtype
+        self.device = torch.device(device)
+        if self.dtype == torch.float32 and self.device.type == "cuda":
+            torch.backends.cuda.matmul.allow_tf32 = False          # float32 means float32 products
+            torch.backends.cudnn.allow_tf32 = False
+        self.ops = make_ops(backend, self.dtype, self.device)
+        self.model = model_cls.from_config(config, weights, self.ops, self.device, self.dtype, page=page)
+        self.cache = PagedCache(self.model.cache_rows, (int(max_tokens) + page - 1) // page, max_seqs, self.dtype, self.device,
+                                page=page)
+        self.scheduler = Scheduler(self.cache, max_batch_tokens, prefill_chunk)
+        self.requests = {}
+        self._ids = itertools.count()
+
+    @classmethod
+    def from_pretrained(cls, model_dir, **kw):
+        """model_dir: config.json + *.safetensors; the model class is chosen by the config's architecture."""
+        from ..loader import iterate_checkpoint
+        config = registry.read_config(model_dir)
+        model_cls, kind = registry.resolve_model(config)
+        if kind != "paged":
+            raise ValueError(f"architecture {registry.architecture_of(config)!r} is served by the {kind} engine, not this one")
+        return cls(model_cls, config, dict(iterate_checkpoint(model_dir)), **kw)
+
+    # ---- the step function -------------------------------------------------------------------------------------------------
+    def open_sequence(self):
+        return self.cache.admit()
+
+    def close_sequence(self, slot):
+        self.cache.release(slot)
+
+    @torch.no_grad()
+    def execute(self, items, want):
+        """items: [(slot, tokens)] - the next tokens of live sequences, all run as one batch; want: flat indices into the
+        concatenated tokens.  -> float logits [len(want), vocab] (None if want is empty)."""
+        toks, seq, pos, rows = [], [], [], []
+        V = self.model.vocab
+        for slot, t in items:
+            start = self.cache.length[slot]
+            if any(not 0 <= int(v) < V for v in t):
+                raise ValueError(f"token id outside the vocabulary of {V}")
+            rows += self.cache.extend(slot, len(t))
+            toks += [int(v) for v in t]
+            seq += [slot] * len(t)
+            pos += range(start, start + len(t))
+        if not toks:
+            return None
+        dev = self.device
+        # (one host tensor, one copy: int64 rows and int32 metadata share a buffer)
+        meta = torch.tensor([toks, seq, pos], dtype=torch.int32).to(dev)
+        batch = StepBatch(tokens=meta[0], seq=meta[1], pos=meta[2], slot=torch.tensor(rows, dtype=torch.int64).to(dev),
+                          block_table=self.cache.block_table(), max_pos=max(pos), n_tokens=len(toks))
+        x = self.model.forward(batch, self.cache.pools)
+        if not want:
+            return None
+        return self.model.logits(x, torch.tensor(list(want), dtype=torch.int32).to(dev))
+
+    # ---- generation ------------------------------------------------------------------------------------------------------------
+    def add_request(self, prompt, params=None, request_id=None):
+        params = params or SamplingParams()
+        rid = request_id if request_id is not None else f"req{next(self._ids)}"
+        r = Request(rid, [int(t) for t in prompt], params)
+        if params.seed is not None:
+            r.generator = torch.Generator(device=self.device).manual_seed(params.seed)
+        self.scheduler.add(r)
+        self.requests[rid] = r
+        return rid
+
+    def step(self):
+        """Run one scheduled batch.  -> [(request id, new token, finished)] for the requests that got a token."""
+        work = self.scheduler.schedule()
+        if not work:
+            return []
+        want, at = [], 0
+        for w in work:
+            at += len(w.tokens)
+            if w.sample:
+                want.append(at - 1)
+        logits = self.execute([(w.request.slot, w.tokens) for w in work], want)
+        for w in work:
+            w.request.computed += len(w.tokens)
+        out = []
+        if want:
+            sampling = [w.request for w in work if w.sample]
+            new = sample(logits, [r.params for r in sampling], [r.generator for r in sampling])
+            for r, tok in zip(sampling, new):
+                r.output.append(tok)
+                done = len(r.output) >= r.params.max_new or (r.params.stop_token is not None and tok == r.params.stop_token)
+                if done:
+                    self.scheduler.finish(r)
+                out.append((r.id, tok, done))
+        return out
+
+    def has_work(self):
+        return bool(self.scheduler.waiting or self.scheduler.running)
+
+    def generate(self, prompts, params=None, **kw):
+        """prompts: lists of token ids -> lists of generated token ids (same order)."""
+        if params is None:
+            params = SamplingParams(**kw)
+        ids = [self.add_request(p, params) for p in prompts]
+        while self.has_work():
+            if not self.step() and not self.scheduler.running:
+                raise RuntimeError("the scheduler cannot place any waiting request")
+        return [self.requests.pop(i).output for i in ids]
