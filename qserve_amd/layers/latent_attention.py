@@ -54,7 +54,7 @@ class LatentAttention:
         qn = q.view(T, H, self.dim + self.rot_dim)[..., :self.dim].transpose(0, 1)  # [H, T, dim] (strided view)
         q_abs = torch.bmm(qn, self.w_uk)                                            # [H, T, rank]
         qf = ops.latent_query(q, q_abs, rope, batch.pos, self.scale, H, self.dim, self.rot_dim, self.rot_n, self.rank)
-        o_lat = ops.latent_attention(qf, pool, batch.block_table, batch.seq, batch.pos, self.window, self.rank, self.page)
+        o_lat = ops.latent_attention(qf, pool, batch, self.window, self.rank, self.page)
         o = torch.bmm(o_lat.transpose(0, 1), self.w_uv_t).transpose(0, 1).reshape(T, H * self.vdim)
         if self.gated:
             ops.sigmoid_gate(o, down[:, self.g_off:self.g_off + H * self.vdim])

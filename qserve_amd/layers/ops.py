@@ -91,11 +91,20 @@ class HipOps:
                    "latent_query")
         return qf
 
-    def latent_attention(self, qf, pool, block_table, seq, pos, window, rank, page, variant=0):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0):
+        """batch: the step's StepBatch (block table, sequence slot and position per token, work tiles).  variant: 0 = the
+        matrix-core kernel where it takes the sizes, 1 = always the wave kernel."""
         T, H, R = qf.shape
+        block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         self._need(qf, pool, block_table, seq, pos)
         assert pool.size(-1) == R and block_table.dtype == torch.int32 and seq.dtype == torch.int32
+        if variant == 0 and self.L.qsv_latent_attention_mfma_ok(rank, R, self.code):
+            tiles = batch.tiles(self.L.qsv_latent_attention_tile_tokens(H))
+            self.check(self.L.qsv_latent_attention_mfma(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
+                                                        block_table.stride(0), pos.data_ptr(), tiles.data_ptr(), tiles.size(0),
+                                                        int(window or 0), H, rank, R, page, self._s()), "latent_attention_mfma")
+            return out
         self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
                                                rank, R, page, self.code, variant, self._s()), "latent_attention")
@@ -191,8 +200,9 @@ class TorchOps:
         qr = _rotate(q.view(T, heads, dim + rot_dim)[..., dim:].float(), rope, pos, rot_n)
         return (torch.cat([q_abs.transpose(0, 1).float(), qr], dim=-1) * scale).contiguous()
 
-    def latent_attention(self, qf, pool, block_table, seq, pos, window, rank, page, variant=0):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0):
         T, H, R = qf.shape
+        block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         bt = block_table.long()
         for t in range(T):

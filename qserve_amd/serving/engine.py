@@ -6,7 +6,7 @@ over it and returns float logits at the rows asked for.  Callers that bring thei
 use `open_sequence` / `execute` / `close_sequence` directly and so drive the very same cache and kernels.
 """
 import itertools
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
@@ -29,6 +29,19 @@ class StepBatch:
     block_table: torch.Tensor   # int32 [slots, pages]
     max_pos: int                # host: largest position in the batch
     n_tokens: int
+    items: list = None          # host: [(sequence slot, first flat token index, tokens)] - runs of consecutive positions
+    _tiles: dict = field(default_factory=dict)
+
+    def tiles(self, tokens_per_tile):
+        """Work tiles for kernels that serve a few consecutive tokens of one sequence per workgroup: int32 [n, 3] =
+        (sequence slot, first flat token index, tokens <= tokens_per_tile), on the device; cached per size."""
+        t = self._tiles.get(tokens_per_tile)
+        if t is None:
+            rows = [(slot, first + o, min(tokens_per_tile, n - o)) for slot, first, n in self.items
+                    for o in range(0, n, tokens_per_tile)]
+            t = torch.tensor(rows, dtype=torch.int32).reshape(-1, 3).to(self.tokens.device if self.tokens is not None else self.pos.device)
+            self._tiles[tokens_per_tile] = t
+        return t
 
 
 class Engine:
@@ -68,10 +81,12 @@ class Engine:
     def execute(self, items, want):
         """items: [(slot, tokens)] - the next tokens of live sequences, all run as one batch; want: flat indices into the
         concatenated tokens.  -> float logits [len(want), vocab] (None if want is empty)."""
-        toks, seq, pos, rows = [], [], [], []
+        toks, seq, pos, rows, runs = [], [], [], [], []
         V = self.model.vocab
         for slot, t in items:
             start = self.cache.length[slot]
+            if len(t):
+                runs.append((slot, len(toks), len(t)))
             if any(not 0 <= int(v) < V for v in t):
                 raise ValueError(f"token id outside the vocabulary of {V}")
             rows += self.cache.extend(slot, len(t))
@@ -84,7 +99,7 @@ class Engine:
         # (one host tensor, one copy: int64 rows and int32 metadata share a buffer)
         meta = torch.tensor([toks, seq, pos], dtype=torch.int32).to(dev)
         batch = StepBatch(tokens=meta[0], seq=meta[1], pos=meta[2], slot=torch.tensor(rows, dtype=torch.int64).to(dev),
-                          block_table=self.cache.block_table(), max_pos=max(pos), n_tokens=len(toks))
+                          block_table=self.cache.block_table(), max_pos=max(pos), n_tokens=len(toks), items=runs)
         x = self.model.forward(batch, self.cache.pools)
         if not want:
             return None
