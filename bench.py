@@ -81,6 +81,10 @@ def parse():
     ap.add_argument("--scaling", default=None, choices=["weak", "strong"],
                     help="N>1 (tensor parallel): weak = --batch sequences PER GPU (global batch = batch x N, so every "
                          "rank keeps N=1's GEMM MACs and KV bytes); strong = --batch is the global batch")
+    ap.add_argument("--design", default=None, choices=["vekalorn"],
+                    help="instead of the default workload: prompt-phase and decode throughput of a design served by the paged "
+                         "engine (qserve_amd/serving) beside the W4A8KV4 Llama engine at equal size; one JSON line per size")
+    ap.add_argument("--design-sizes", default="w2048,w4096", help="with --design: comma-separated size names (qserve_amd/serving/bench.py)")
     a = ap.parse_args()
     preset = CONFIGS[a.config] if a.config else CONFIGS[2]
     for k, v in preset.items():
@@ -517,6 +521,9 @@ def cpu_baseline(args, cfg, torch):
 
 def main():
     args = parse()
+    if args.design:
+        from qserve_amd.serving import bench as design_bench
+        sys.exit(design_bench.main(args, sys.modules[__name__]))
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ and "RANK" not in os.environ:
         sys.exit(self_launch(args))
     import torch

@@ -81,6 +81,16 @@ int qsv_moe_up(void* act, const void* h, const void* up, const int32_t* idx, int
 int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx, const float* weight, int n_tokens,
                  int top_k, int width, int ff, int dtype, void* stream);
 
+/* Expert-sorted form for many tokens: slots (t, k) are sorted by expert on the host side of the ABI, the expert products run
+ * as ordinary matrix products over contiguous runs of sorted slots, and these kernels do the rest:
+ *   out[i] = src[order[i] / div]                                   (rows into sorted order)
+ *   a[i]   = relu(a[i])^2                                           (in place)
+ *   y[t]   = sum_k weight[t, k] * ys[inv[t * top_k + k]]            (sorted rows back, weighted; float accumulation) */
+int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, int n_rows, int width, int dtype, void* stream);
+int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream);
+int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n_tokens, int top_k, int width,
+                    int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -107,7 +107,63 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(T* __restrict__ y, const T
         if (lane == 0) st(y, t * D + d, total);
     }
 }
+
+// ---- expert-sorted form (many tokens): the products are the vendor's, per expert over contiguous runs of sorted slots; these
+// kernels do the permutation in, the activation, and the weighted permutation out -----------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(NT) void gather_rows_kernel(T* __restrict__ out, const T* __restrict__ src,
+                                                         const int64_t* __restrict__ order, int div, int width) {
+    const size_t i = blockIdx.x;
+    const T* s = src + (size_t)(order[i] / div) * width;
+    for (int c = threadIdx.x; c < width; c += NT) out[i * width + c] = s[c];
+}
+template <typename T>
+__global__ __launch_bounds__(NT) void relu_sq_kernel(T* __restrict__ a, size_t n) {
+    const size_t i = (size_t)blockIdx.x * NT + threadIdx.x;
+    if (i < n) {
+        const float v = fmaxf(ld(a, i), 0.f);
+        st(a, i, v * v);
+    }
+}
+// y[t] = sum_k weight[t, k] * ys[inv[t top_k + k]]
+template <typename T>
+__global__ __launch_bounds__(NT) void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ ys, const int64_t* __restrict__ inv,
+                                                         const float* __restrict__ weight, int top_k, int D) {
+    const size_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < D; c += NT) {
+        float a = 0.f;
+        for (int k = 0; k < top_k; ++k) a += weight[t * top_k + k] * ld(ys, (size_t)inv[t * top_k + k] * D + c);
+        st(y, t * D + c, a);
+    }
+}
 }  // namespace
+
+extern "C" int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, int n_rows, int width, int dtype,
+                               void* stream) {
+    QSV_REQUIRE(out && src && order && div > 0 && n_rows >= 0 && width > 0, "qsv_gather_rows: bad arguments");
+    if (n_rows == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_gather_rows",
+                 hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(n_rows), dim3(NT), 0, (hipStream_t)stream, (T*)out, (const T*)src,
+                                    order, div, width));
+    return qsv_launch_status("qsv_gather_rows");
+}
+extern "C" int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream) {
+    QSV_REQUIRE(a && n >= 0 && n < (1ll << 31) * NT, "qsv_relu_sq: bad arguments");
+    if (n == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_relu_sq",
+                 hipLaunchKernelGGL(relu_sq_kernel<T>, dim3((unsigned)((n + NT - 1) / NT)), dim3(NT), 0, (hipStream_t)stream, (T*)a,
+                                    (size_t)n));
+    return qsv_launch_status("qsv_relu_sq");
+}
+extern "C" int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n, int top_k, int D,
+                               int dtype, void* stream) {
+    QSV_REQUIRE(y && ys && inv && weight && n >= 0 && top_k > 0 && D > 0, "qsv_moe_combine: bad arguments");
+    if (n == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_moe_combine",
+                 hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, (T*)y, (const T*)ys, inv,
+                                    weight, top_k, D));
+    return qsv_launch_status("qsv_moe_combine");
+}
 
 extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, int n, int D, int E, int top_k,
                              int G, int keep, int dtype, void* stream) {

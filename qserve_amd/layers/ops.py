@@ -131,6 +131,8 @@ class HipOps:
         """up [E, ff, D], down [E, D, ff]; y[t] = sum_k wt[t, k] * down[idx[t, k]] relu(up[idx[t, k]] h[t])^2."""
         T, D = h.shape
         top_k, ff = idx.size(1), up.size(1)
+        if T * top_k > self.moe_sorted_above:
+            return self._moe_experts_sorted(h, up, down, idx, wt)
         act = torch.empty((T, top_k, ff), dtype=self.dtype, device=h.device)
         y = torch.empty((T, D), dtype=self.dtype, device=h.device)
         self._need(h, up, down, idx, wt)
@@ -139,6 +141,41 @@ class HipOps:
                                      self._s()), "moe_up")
         self.check(self.L.qsv_moe_down(y.data_ptr(), act.data_ptr(), down.data_ptr(), idx.data_ptr(), wt.data_ptr(), T, top_k, D,
                                        ff, self.code, self._s()), "moe_down")
+        return y
+
+
+    # More (token, expert) slots than this: sort the slots by expert and run each expert as one matrix product.  Below it the
+    # per-token kernels above are used: no host synchronisation, a fixed launch sequence.
+    moe_sorted_above = 64
+
+    def _moe_experts_sorted(self, h, up, down, idx, wt):
+        T, D = h.shape
+        E, ff, K = up.size(0), up.size(1), idx.size(1)
+        n = T * K
+        flat = idx.reshape(-1)
+        order = torch.argsort(flat, stable=True)                       # sorted slot -> slot (t K + k)
+        counts = torch.bincount(flat, minlength=E).tolist()            # (host synchronisation: the runs' lengths)
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(n, device=h.device)                  # slot -> sorted slot
+        xs = torch.empty((n, D), dtype=self.dtype, device=h.device)
+        self.check(self.L.qsv_gather_rows(xs.data_ptr(), h.data_ptr(), order.data_ptr(), K, n, D, self.code, self._s()),
+                   "gather_rows")
+        act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
+        ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
+        a = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.matmul(xs[a:a + c], up[e].t(), out=act[a:a + c])
+            a += c
+        self.check(self.L.qsv_relu_sq(act.data_ptr(), act.numel(), self.code, self._s()), "relu_sq")
+        a = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.matmul(act[a:a + c], down[e].t(), out=ys[a:a + c])
+            a += c
+        y = torch.empty((T, D), dtype=self.dtype, device=h.device)
+        self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
+                                          self._s()), "moe_combine")
         return y
 
 

@@ -1,0 +1,231 @@
+"""Throughput of a served design at layer sizes of real models, beside the W4A8KV4 Llama engine at equal size.
+
+    python bench.py --design vekalorn [--design-sizes w2048,w4096] [--steps K] [--warmup W]
+
+Per size (random weights, 4 layers, vocabulary 32000): prompt phase = 8 prompts x 1024 tokens in one step through
+Engine.execute; decoding = 64 sequences at context 1024, one token each per step.  Beside them the Llama-style W4A8KV4
+engine (qserve_amd.decode.DecodeEngine) with the same width, head count and ACTIVE feed-forward width, same batch and
+context.  Per kernel class the achieved fraction of its roofline (HBM bytes for decoding, dense bf16 / fp16 matrix-core
+peak for the prompt phase) is printed for both, from HIP events around every launch of one step.
+One JSON line per size on standard output.
+"""
+import json
+import math
+import time
+
+import torch
+
+BF16_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+SIZES = {
+    "w2048": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, window=1024,
+                  experts=16, groups=4, keep=2, top=4, ff=1408),
+    "w4096": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=1536, window=1024,
+                  experts=32, groups=8, keep=4, top=4, ff=2752),
+}
+LAYERS, VOCAB = 4, 32000
+
+
+def vekalorn_config(s):
+    rot = {"base": 10000.0, "dims": s["rot_dim"], "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"]},
+           "router": {"experts": s["experts"], "top": s["top"], "groups": {"count": s["groups"], "keep": s["keep"]}}}
+    common = {k: s[k] for k in ("heads", "dim", "vdim", "kv_rank", "q_rank")}
+    a2 = {"type": "latent_attention_2", "mlp": mlp,
+          "mixer": dict(common, rot_dim=s["rot_dim"], rot=rot, scale=1.0 / math.sqrt(s["dim"] + s["rot_dim"]))}
+    a1 = {"type": "latent_attention", "mlp": mlp,
+          "mixer": dict(common, mask={"size": s["window"]}, scale=1.0 / math.sqrt(s["dim"]))}
+    return {"architecture": "Vekalorn", "width": s["width"], "vocab": VOCAB, "norm": {"eps": 1e-5},
+            "layers": [a2, a1, a1, a2][:LAYERS]}
+
+
+def random_weights(cfg, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+
+    def mat(o, i, s=1.0):
+        return (torch.randn((o, i), device=dev, generator=g) * (s / math.sqrt(i))).bfloat16()
+
+    def vec(n):
+        return (1.0 + 0.1 * torch.randn((n,), device=dev, generator=g)).bfloat16()
+
+    W = {"embed": torch.randn((V, D), device=dev, generator=g).bfloat16(), "head": mat(V, D), "final.norm": vec(D)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        H, d, dv, r, qr = m["heads"], m["dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+        dr = m.get("rot_dim", 0)
+        W[p + "norm1"], W[p + "norm2"] = vec(D), vec(D)
+        W[p + "mix.dq"], W[p + "mix.dq.norm"], W[p + "mix.uq"] = mat(qr, D), vec(qr), mat(H * (d + dr), qr)
+        W[p + "mix.dkv"], W[p + "mix.dkv.norm"] = mat(r + dr, D), vec(r)
+        W[p + "mix.uk"], W[p + "mix.uv"], W[p + "mix.o"] = mat(H * d, r), mat(H * dv, r), mat(D, H * dv)
+        if L["type"] == "latent_attention_2":
+            W[p + "mix.g"] = mat(H * dv, D)
+        E, ff = L["mlp"]["router"]["experts"], L["mlp"]["expert"]["ff"]
+        for e in range(E):
+            W[f"{p}mlp.e{e}.up"], W[f"{p}mlp.e{e}.down"] = mat(ff, D), mat(D, ff)
+        W[p + "mlp.router"] = mat(E, D, 3.0)
+    return W
+
+
+class OpTimer:
+    """HIP events around every call of the ops object's methods and of the vendor products (one step at a time)."""
+    NAMES = ("embed", "add_layer_norm", "layer_norm_rows", "latent_prep", "latent_query", "latent_attention", "sigmoid_gate",
+             "moe_route", "moe_experts")
+
+    def __init__(self, ops):
+        self.ops, self.events, self.on = ops, [], False
+        for n in self.NAMES:
+            setattr(ops, n, self._wrap(n, getattr(ops, n)))
+
+    def _wrap(self, name, fn):
+        def timed(*a, **k):
+            if not self.on:
+                return fn(*a, **k)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            self.events.append((name, e0, e1))
+            return r
+        return timed
+
+    def step(self, fn):
+        """Run fn() with timing on -> ({op: ms summed over its launches}, total ms between first and last event)."""
+        self.events, self.on = [], True
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        fn()
+        t1.record()
+        self.on = False
+        torch.cuda.synchronize()
+        out = {}
+        for n, e0, e1 in self.events:
+            out[n] = out.get(n, 0.0) + e0.elapsed_time(e1)
+        return out, t0.elapsed_time(t1)
+
+
+def timed(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def bench_vekalorn(name, s, dev, steps, warmup):
+    from ..models.vekalorn import Vekalorn
+    from .engine import Engine
+    cfg = vekalorn_config(s)
+    NB, L, BP = 64, 1024, 8
+    eng = Engine(Vekalorn, cfg, random_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 64), max_seqs=NB)
+    timer = OpTimer(eng.ops)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, VOCAB, (L,), generator=g).tolist() for _ in range(NB)]
+    slots = [eng.open_sequence() for _ in range(NB)]
+    # prompt phase: 8 steps of 8 prompts (fills the cache for decoding); step 0 warms up, the others are timed
+    pre_ms, ops_pre = [], None
+    for i in range(0, NB, BP):
+        items = [(slots[j], prompts[j]) for j in range(i, i + BP)]
+        want = [k * L + L - 1 for k in range(BP)]
+        if i == BP:                                          # one step with events around every launch
+            ops_pre, _ = timer.step(lambda: eng.execute(items, want))
+            continue
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.execute(items, want)
+        torch.cuda.synchronize()
+        if i > 0:
+            pre_ms.append((time.perf_counter() - t0) * 1e3)
+    pre = sorted(pre_ms)[len(pre_ms) // 2]
+    # decoding
+    nxt = [[int(torch.randint(0, VOCAB, (1,), generator=g))] for _ in range(NB)]
+    want = list(range(NB))
+
+    def decode():
+        eng.execute([(slots[j], nxt[j]) for j in range(NB)], want)
+
+    res = {}
+    for label, above in (("sorted_experts", 0), ("per_token_experts", 10 ** 9)):
+        eng.ops.moe_sorted_above = above
+        res[label] = timed(decode, steps, warmup)
+    del eng.ops.moe_sorted_above
+    dec = timed(decode, steps, warmup)
+    ops_dec, dec_events_ms = timer.step(decode)
+    ctx = eng.cache.length[slots[0]]
+    # rooflines
+    m1 = cfg["layers"][1]["mixer"]
+    H, rank = m1["heads"], m1["kv_rank"]
+    rows = {"latent_attention_2": rank + s["rot_dim"], "latent_attention": rank}
+    kinds = [x["type"] for x in cfg["layers"]]
+    T = BP * L
+    flops = sum(sum(min(p + 1, s["window"]) if k == "latent_attention" else p + 1 for p in range(L)) * BP * H * (rows[k] + rank) * 2.0
+                for k in kinds)
+    att_pre = flops / (ops_pre["latent_attention"] * 1e-3) / 1e12
+    by = sum(NB * (min(ctx, s["window"]) if k == "latent_attention" else ctx) * rows[k] * 2.0 for k in kinds)
+    att_dec = by / (ops_dec["latent_attention"] * 1e-3) / 1e9
+    moe_flops = LAYERS * T * s["top"] * 2 * 2.0 * s["ff"] * s["width"]
+    moe_pre = moe_flops / (ops_pre["moe_experts"] * 1e-3) / 1e12
+    moe_bytes = LAYERS * min(s["experts"], NB * s["top"]) * 2 * s["ff"] * s["width"] * 2.0
+    moe_dec = moe_bytes / (ops_dec["moe_experts"] * 1e-3) / 1e9
+    out = dict(model=f"Vekalorn-{name}", prefill_tokens_per_s=T / pre * 1e3, prefill_ms=pre, decode_tokens_per_s=NB / dec * 1e3,
+               decode_ms=dec, decode_ms_by_expert_form=res, decode_ms_gpu_events=dec_events_ms, context=ctx,
+               prefill_ops_ms=ops_pre, decode_ops_ms=ops_dec,
+               roofline=dict(prefill_attention_tflops=att_pre, prefill_attention_frac_bf16_peak=att_pre / BF16_PEAK_TFLOPS,
+                             decode_attention_gbs=att_dec, decode_attention_frac_hbm=att_dec / HBM_PEAK_GBS,
+                             prefill_experts_tflops=moe_pre, prefill_experts_frac_bf16_peak=moe_pre / BF16_PEAK_TFLOPS,
+                             decode_experts_gbs=moe_dec, decode_experts_frac_hbm=moe_dec / HBM_PEAK_GBS))
+    for sl in slots:
+        eng.close_sequence(sl)
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_llama(name, s, dev, steps, warmup, helpers):
+    """The closest existing model at equal size: same width and heads (head dimension 128), feed-forward width = the active
+    expert width, W4A8 per-channel weights, KV4 cache."""
+    from .. import decode as D
+    cfg = dict(name=f"llama-w4a8-{name}", hidden=s["width"], heads=s["heads"], kv_heads=s["heads"], inter=s["top"] * s["ff"],
+               layers=LAYERS, vocab=VOCAB, rope_theta=1e4, eps=1e-5)
+    NB, L, BP = 64, 1024, 8
+    pe = D.DecodeEngine(cfg, batch=BP, prompt_len=L, max_new=8, device=dev)
+    pre = timed(lambda: pe.prefill(L), 3, 1)
+    del pe
+    torch.cuda.empty_cache()
+    eng = D.DecodeEngine(cfg, batch=NB, prompt_len=L, max_new=64, device=dev)
+    eng.prefill_cache(L)
+    eager = timed(eng.step, steps, warmup)
+    eng.lengths.fill_(L + 1)
+    eng.capture()
+    dec = timed(eng.run, steps, warmup)
+    eng.lengths.fill_(L + 1)
+    ns = type("A", (), {})()
+    kern = helpers.kernel_bench(eng, ns, torch, [L + 1]) + helpers.prefill_attention_bench(torch, dev, cfg, BP, L)
+    keep = [{k: v for k, v in r.items() if k in ("kernel", "us", "gbs", "tops", "tflops", "frac_of_hbm_peak", "frac_of_fp16_mfma_peak")}
+            for r in kern]
+    gemm = [r for r in kern if r.get("family") == "w4a8_gemm"]
+    return dict(model=cfg["name"], prefill_tokens_per_s=BP * L / pre * 1e3, prefill_ms=pre, decode_tokens_per_s=NB / dec * 1e3,
+                decode_ms=dec, decode_ms_eager=eager, kernels=keep,
+                roofline=dict(decode_gemm_frac_hbm=sum(r["bytes"] for r in gemm) / sum(r["us"] for r in gemm) / 1e3 / HBM_PEAK_GBS))
+
+
+def main(args, helpers):
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    from .. import build
+    import os
+    if not os.path.exists(build.LIB):
+        build.build(verbose=False)
+    steps, warmup = min(args.steps, 32), min(args.warmup, 8)
+    for name in args.design_sizes.split(","):
+        s = SIZES[name]
+        line = {"design": args.design, "size": name, "sizes": s, "layers": LAYERS, "vocab": VOCAB, "dtype": "bf16",
+                "data": "synthetic", "workload": "prefill 8 x 1024 tokens in one step; decode 64 sequences at context 1024"}
+        line["vekalorn"] = bench_vekalorn(name, s, dev, steps, warmup)
+        line["llama_w4a8"] = bench_llama(name, s, dev, steps, warmup, helpers)
+        print(json.dumps(line), flush=True)
+    return 0

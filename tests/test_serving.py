@@ -211,6 +211,12 @@ def test_router_and_experts_alone(backend):
         y = ops.moe_experts(h.to(dev), torch.stack(ups).to(dev), torch.stack(downs).to(dev), idx, wt)
         ref = P.moe(h.double(), W, "p.", {"router": r})
         assert_close(y.double().cpu(), ref, 1e-5, f"moe E={E}")
+        if backend == "hip":                                  # both forms: per-token kernels and expert-sorted products
+            for above in (0, 10 ** 9):
+                ops.moe_sorted_above = above
+                y = ops.moe_experts(h.to(dev), torch.stack(ups).to(dev), torch.stack(downs).to(dev), idx, wt)
+                assert_close(y.double().cpu(), ref, 1e-5, f"moe E={E}, sorted above {above}")
+            del ops.moe_sorted_above
 
 
 def test_group_limit_changes_the_choice(backend):
