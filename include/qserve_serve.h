@@ -54,15 +54,18 @@ int qsv_latent_attention(void* out, const float* qf, const void* pool, const int
                          const int32_t* seq, const int32_t* pos, int window, int n_tokens, int heads, int rank,
                          int row_width, int page, int dtype, int variant, void* stream);
 
+int qsv_latent_attention_tile_tokens(int heads);
+int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
 /* The same attention on the bf16 matrix cores.  The host cuts every sequence's tokens of the step into work tiles of at most
  * qsv_latent_attention_tile_tokens(heads) consecutive tokens: tiles int32 [n_tiles, 3] = (sequence slot, first flat token
  * index, tokens).  qsv_latent_attention_mfma_ok() says whether the sizes are taken (bfloat16 storage, rank and row width
- * multiples of 8, row width <= 576); otherwise use qsv_latent_attention. */
-int qsv_latent_attention_tile_tokens(int heads);
-int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
+ * multiples of 8, row width <= 576); otherwise use qsv_latent_attention. * key_splits > 1 cuts every tile's keys over that many workgroups and merges the partial results in a second launch (steps
+ * with few tiles: decoding); part_o (float [key_splits, n_tokens, heads, rank]) and part_ml (float [key_splits, n_tokens,
+ * heads, 2]) are its workspace. */
 int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                               const int32_t* pos, const int32_t* tiles, int n_tiles, int window, int heads, int rank,
-                              int row_width, int page, void* stream);
+                              int row_width, int page, int key_splits, float* part_o, float* part_ml, int n_tokens,
+                              void* stream);
 
 /* o[t, i] *= sigmoid(g[t * g_stride + i]),  i < n. */
 int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int n, int dtype, void* stream);

@@ -91,19 +91,32 @@ class HipOps:
                    "latent_query")
         return qf
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0):
+    attention_split_target = 512        # workgroups a launch of the matrix-core attention should at least have
+
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None):
         """batch: the step's StepBatch (block table, sequence slot and position per token, work tiles).  variant: 0 = the
-        matrix-core kernel where it takes the sizes, 1 = always the wave kernel."""
+        matrix-core kernel where it takes the sizes, 1 = always the wave kernel.  key_splits: None = chosen from the number
+        of workgroups and the context."""
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         self._need(qf, pool, block_table, seq, pos)
         assert pool.size(-1) == R and block_table.dtype == torch.int32 and seq.dtype == torch.int32
-        if variant == 0 and self.L.qsv_latent_attention_mfma_ok(rank, R, self.code):
+        if variant == 0 and page % 32 == 0 and self.L.qsv_latent_attention_mfma_ok(rank, R, self.code):
             tiles = batch.tiles(self.L.qsv_latent_attention_tile_tokens(H))
+            # few workgroups and long contexts (decoding): cut the keys over several workgroups, merged by a second launch
+            groups = tiles.size(0) * ((H + 31) // 32)
+            span = min(batch.max_pos + 1, int(window)) if window else batch.max_pos + 1
+            splits = max(1, min(self.attention_split_target // max(groups, 1), span // 128, 32)) if key_splits is None else key_splits
+            po = pm = None
+            if splits > 1:
+                po = torch.empty((splits, T, H, rank), dtype=torch.float32, device=qf.device)
+                pm = torch.empty((splits, T, H, 2), dtype=torch.float32, device=qf.device)
             self.check(self.L.qsv_latent_attention_mfma(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                         block_table.stride(0), pos.data_ptr(), tiles.data_ptr(), tiles.size(0),
-                                                        int(window or 0), H, rank, R, page, self._s()), "latent_attention_mfma")
+                                                        int(window or 0), H, rank, R, page, splits,
+                                                        0 if po is None else po.data_ptr(), 0 if pm is None else pm.data_ptr(), T,
+                                                        self._s()), "latent_attention_mfma")
             return out
         self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
@@ -237,7 +250,7 @@ class TorchOps:
         qr = _rotate(q.view(T, heads, dim + rot_dim)[..., dim:].float(), rope, pos, rot_n)
         return (torch.cat([q_abs.transpose(0, 1).float(), qr], dim=-1) * scale).contiguous()
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None):
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)

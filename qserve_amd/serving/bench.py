@@ -21,6 +21,8 @@ HBM_PEAK_GBS = 8000.0
 SIZES = {
     "w2048": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, window=1024,
                   experts=16, groups=4, keep=2, top=4, ff=1408),
+    "w2048r256": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=256, q_rank=768, window=1024,
+                      experts=16, groups=4, keep=2, top=4, ff=1408),
     "w4096": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=1536, window=1024,
                   experts=32, groups=8, keep=4, top=4, ff=2752),
 }
@@ -121,7 +123,7 @@ def bench_vekalorn(name, s, dev, steps, warmup):
     from .engine import Engine
     cfg = vekalorn_config(s)
     NB, L, BP = 64, 1024, 8
-    eng = Engine(Vekalorn, cfg, random_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 64), max_seqs=NB)
+    eng = Engine(Vekalorn, cfg, random_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 256), max_seqs=NB)
     timer = OpTimer(eng.ops)
     g = torch.Generator().manual_seed(1)
     prompts = [torch.randint(0, VOCAB, (L,), generator=g).tolist() for _ in range(NB)]

@@ -70,3 +70,44 @@ def test_product_does_not_import_oracle():
                     if re.search(r"^\s*(from|import)\s+oracle\b", open(os.path.join(dp, f)).read(), flags=re.M):
                         bad.append(os.path.join(dp, f))
     assert not bad, f"product code imports the oracle: {bad}"
+
+
+# ---- libqserve_serve.so (include/qserve_serve.h): the paged serving engine's kernels ----------------------------------------------
+
+def serve_header_symbols():
+    txt = open(os.path.join(ROOT, "include", "qserve_serve.h")).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(qsv_[a-z0-9_]+)\s*\(", txt)))
+
+
+def test_serve_library_builds_and_matches_its_header():
+    from qserve_amd import build
+    from qserve_amd.serving import _lib
+    lib = ctypes.CDLL(build.build_serve(verbose=False))
+    for s in serve_header_symbols():
+        assert hasattr(lib, s), f"{s} declared in include/qserve_serve.h but not exported"
+    assert sorted(_lib.SIGNATURES) == serve_header_symbols()
+    assert _lib.lib().qsv_arch() == b"gfx950"
+
+
+def test_serve_argument_validation_without_gpu():
+    from qserve_amd.serving._lib import check, lib
+    L = lib()
+    assert L.qsv_moe_route(1, 1, 1, 1, 4, 64, 8, 3, 4, 1, 0, None) == 1          # top 3 of one kept group of 2
+    assert b"experts" in L.qsv_last_error()
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 600, 640, 64, 0, 1, None) == 1   # rows wider than 576
+    assert L.qsv_latent_attention_mfma_ok(96, 112, 0) == 1 and L.qsv_latent_attention_mfma_ok(96, 112, 1) == 0
+    assert L.qsv_latent_attention_mfma_ok(70, 70, 0) == 0
+    assert [L.qsv_latent_attention_tile_tokens(h) for h in (1, 3, 6, 16, 32, 40)] == [64, 16, 8, 4, 4, 4]
+    with pytest.raises(RuntimeError):
+        check(L.qsv_embed(0, 1, 1, 1, 1, 8, 0, None), "embed")
+
+
+def test_serving_package_does_not_need_the_w4a8_library():
+    """Importing the serving engine (and replaying a trace) must not load libqserve_amd.so: a fresh checkout builds only
+    the serving kernels."""
+    import subprocess
+    import sys
+    code = ("import sys; import qserve_amd.serving, qserve_amd.models.vekalorn, qserve_amd.serving.trace; "
+            "bad = [m for m in sys.modules if m in ('qserve_amd._lib', 'qserve_amd.decode', 'qserve_backend')]; sys.exit(1 if bad else 0)")
+    assert subprocess.run([sys.executable, "-c", code], cwd=ROOT).returncode == 0

@@ -586,3 +586,6 @@ def test_matrix_core_attention_matches_the_wave_kernel(heads, rank, rot):
             ref[t] = torch.softmax(qf[t].double() @ rows.T, dim=-1) @ rows[:, :rank]
         assert_close(o_wave, ref, 5e-3, f"wave kernel, window {window}")
         assert_close(o_mfma, ref, 1e-2, f"matrix-core kernel, window {window}")
+        for splits in (1, 3, 8):                                         # the keys of every tile cut over several workgroups
+            o = ops.latent_attention(qf.to(dev), pool.to(dev), b, window, rank, page, key_splits=splits).double().cpu()
+            assert_close(o, ref, 1e-2, f"matrix-core kernel, window {window}, {splits} key splits")
