@@ -108,6 +108,100 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(T* __restrict__ y, const T
     }
 }
 
+// The same two kernels for widths that are multiples of 8: 16-byte weight loads and four output rows per wave in flight at once
+// (the scalar forms above wait for one row's loads before they issue the next row's: latency-bound at real layer sizes).
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 u = *(const uint4*)p;
+    const unsigned w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+constexpr int ROWS = 4;      // output rows a wave works on at once
+
+template <typename T>
+__global__ __launch_bounds__(NT) void moe_up_vec_kernel(T* __restrict__ act, const T* __restrict__ h, const T* __restrict__ up,
+                                                        const int32_t* __restrict__ idx, int top_k, int D, int ff) {
+    extern __shared__ float xs[];
+    const size_t slot = blockIdx.x;
+    const size_t t = slot / top_k;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < D; i += NT) xs[i] = ld(h, t * D + i);
+    __syncthreads();
+    const T* W = up + (size_t)idx[slot] * ff * D;
+    for (int f0 = w * ROWS; f0 < ff; f0 += NW * ROWS) {
+        float acc[ROWS] = {0.f, 0.f, 0.f, 0.f};
+        for (int c = lane * 8; c < D; c += 64 * 8) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = xs[c + e];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                if (f0 + r < ff) {
+                    float v[8];
+                    load8(W + (size_t)(f0 + r) * D + c, v);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[r] += v[e] * x[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const float d = wave_sum(acc[r]);
+            if (lane == 0 && f0 + r < ff) {
+                const float a = fmaxf(d, 0.f);
+                st(act, slot * ff + f0 + r, a * a);
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void moe_down_vec_kernel(T* __restrict__ y, const T* __restrict__ act, const T* __restrict__ down,
+                                                          const int32_t* __restrict__ idx, const float* __restrict__ weight,
+                                                          int top_k, int D, int ff) {
+    extern __shared__ float as[];
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < top_k * ff; i += NT) as[i] = ld(act, t * top_k * ff + i);
+    __syncthreads();
+    for (int d0 = w * ROWS; d0 < D; d0 += NW * ROWS) {
+        float acc[ROWS] = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < top_k; ++k) {
+            const T* Wk = down + (size_t)idx[t * top_k + k] * D * ff;
+            const float wk = weight[t * top_k + k];
+            float part[ROWS] = {0.f, 0.f, 0.f, 0.f};
+            for (int c = lane * 8; c < ff; c += 64 * 8) {
+                float x[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = as[k * ff + c + e];
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    if (d0 + r < D) {
+                        float v[8];
+                        load8(Wk + (size_t)(d0 + r) * ff + c, v);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) part[r] += v[e] * x[e];
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[r] += wk * part[r];
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const float v = wave_sum(acc[r]);
+            if (lane == 0 && d0 + r < D) st(y, t * D + d0 + r, v);
+        }
+    }
+}
+
 // ---- expert-sorted form (many tokens): the products are the vendor's, per expert over contiguous runs of sorted slots; these
 // kernels do the permutation in, the activation, and the weighted permutation out -----------------------------------------------
 template <typename T>
@@ -183,9 +277,14 @@ extern "C" int qsv_moe_up(void* act, const void* h, const void* up, const int32_
     QSV_REQUIRE(act && h && up && idx && n >= 0 && top_k > 0 && D > 0 && ff > 0, "qsv_moe_up: bad arguments");
     QSV_REQUIRE((size_t)D * 4 <= 64 * 1024, "qsv_moe_up: width %d does not fit the workgroup's LDS", D);
     if (n == 0) return QSV_OK;
-    QSV_DISPATCH(dtype, "qsv_moe_up",
-                 hipLaunchKernelGGL(moe_up_kernel<T>, dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,
-                                    (const T*)h, (const T*)up, idx, top_k, D, ff));
+    if (D % 8 == 0)
+        QSV_DISPATCH(dtype, "qsv_moe_up",
+                     hipLaunchKernelGGL(moe_up_vec_kernel<T>, dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,
+                                        (const T*)h, (const T*)up, idx, top_k, D, ff));
+    else
+        QSV_DISPATCH(dtype, "qsv_moe_up",
+                     hipLaunchKernelGGL(moe_up_kernel<T>, dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,
+                                        (const T*)h, (const T*)up, idx, top_k, D, ff));
     return qsv_launch_status("qsv_moe_up");
 }
 
@@ -194,8 +293,13 @@ extern "C" int qsv_moe_down(void* y, const void* act, const void* down, const in
     QSV_REQUIRE(y && act && down && idx && weight && n >= 0 && top_k > 0 && D > 0 && ff > 0, "qsv_moe_down: bad arguments");
     QSV_REQUIRE((size_t)top_k * ff * 4 <= 64 * 1024, "qsv_moe_down: %d x %d activations do not fit the workgroup's LDS", top_k, ff);
     if (n == 0) return QSV_OK;
-    QSV_DISPATCH(dtype, "qsv_moe_down",
-                 hipLaunchKernelGGL(moe_down_kernel<T>, dim3(n), dim3(NT), (size_t)top_k * ff * 4, (hipStream_t)stream, (T*)y,
-                                    (const T*)act, (const T*)down, idx, weight, top_k, D, ff));
+    if (ff % 8 == 0)
+        QSV_DISPATCH(dtype, "qsv_moe_down",
+                     hipLaunchKernelGGL(moe_down_vec_kernel<T>, dim3(n), dim3(NT), (size_t)top_k * ff * 4, (hipStream_t)stream, (T*)y,
+                                        (const T*)act, (const T*)down, idx, weight, top_k, D, ff));
+    else
+        QSV_DISPATCH(dtype, "qsv_moe_down",
+                     hipLaunchKernelGGL(moe_down_kernel<T>, dim3(n), dim3(NT), (size_t)top_k * ff * 4, (hipStream_t)stream, (T*)y,
+                                        (const T*)act, (const T*)down, idx, weight, top_k, D, ff));
     return qsv_launch_status("qsv_moe_down");
 }

@@ -191,8 +191,9 @@ def test_router_and_experts_alone(backend):
     dev = device_of(backend)
     ops = make_ops(backend, torch.float32, dev)
     g = torch.Generator().manual_seed(11)
-    for E, G, keep, top, ff in ((6, 3, 2, 3, 20), (4, 1, 1, 1, 12), (8, 2, 1, 4, 7), (12, 4, 3, 4, 9), (5, 5, 2, 2, 6)):
-        D, T = 40, 33
+    for E, G, keep, top, ff, D in ((6, 3, 2, 3, 20, 40), (4, 1, 1, 1, 12, 40), (8, 2, 1, 4, 7, 36), (12, 4, 3, 4, 9, 40),
+                                   (5, 5, 2, 2, 6, 20), (4, 2, 1, 2, 24, 72), (3, 1, 1, 2, 1032, 520)):
+        T = 33
         h = torch.randn(T, D, generator=g)
         Wr = torch.randn(E, D, generator=g) * 0.6
         r = {"experts": E, "top": top, "groups": {"count": G, "keep": keep}}
