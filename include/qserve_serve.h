@@ -89,6 +89,11 @@ int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx,
  *   out[i] = src[order[i] / div]                                   (rows into sorted order)
  *   a[i]   = relu(a[i])^2                                           (in place)
  *   y[t]   = sum_k weight[t, k] * ys[inv[t * top_k + k]]            (sorted rows back, weighted; float accumulation) */
+/* Expert-major form (bfloat16): out[s, r] = act(W[e][r, :] . X[x_index ? x_index[s] / div : s, :]) for the sorted slots
+ * s in [offsets[e], offsets[e + 1]) of every expert e; W [n_experts, rows, K]; act = relu^2 (relu_sq != 0) or none.  Every
+ * weight is read once per launch.  K a multiple of 8, at most 4096. */
+int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
+                    int n_experts, int rows, int K, int relu_sq, void* stream);
 int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, int n_rows, int width, int dtype, void* stream);
 int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream);
 int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n_tokens, int top_k, int width,

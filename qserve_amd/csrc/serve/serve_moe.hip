@@ -202,6 +202,74 @@ __global__ __launch_bounds__(NT) void moe_down_vec_kernel(T* __restrict__ y, con
     }
 }
 
+// ---- expert-major form (decoding and short portions, bfloat16): slots sorted by expert ON THE DEVICE, workgroup = (16 output rows,
+// expert); a wave keeps its four weight rows in registers (packed bfloat16) and walks the tokens routed to the expert, so every
+// weight is read once per step however many tokens share the expert.  No host synchronisation. ----------------------------------
+template <int KI, bool RELU_SQ>
+__global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
+                                                         const int64_t* __restrict__ x_index, int div, const bf16_t* __restrict__ W,
+                                                         const int64_t* __restrict__ offsets, int rows, int K) {
+    const int e = blockIdx.y;
+    const int64_t s0 = offsets[e], s1 = offsets[e + 1];
+    if (s0 == s1) return;                                                   // nobody chose this expert
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int r0 = (blockIdx.x * NW + w) * ROWS;
+    if (r0 >= rows) return;
+    uint4 wr[ROWS][KI];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const int c = (lane + 64 * i) * 8;
+            wr[r][i] = (r0 + r < rows && c < K) ? *(const uint4*)(W + ((size_t)e * rows + r0 + r) * K + c) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    // TOK tokens at a time: their input pieces are all requested before the first is used (a token at a time, every token
+    // paid a full memory round trip with nothing else in flight)
+    constexpr int TOK = 4;
+    for (int64_t sb = s0; sb < s1; sb += TOK) {
+        uint4 xr[TOK][KI];
+#pragma unroll
+        for (int j = 0; j < TOK; ++j) {
+            const int64_t s = sb + j < s1 ? sb + j : s1 - 1;
+            const bf16_t* x = X + (size_t)(x_index ? x_index[s] / div : s) * K;
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const int c = (lane + 64 * i) * 8;
+                xr[j][i] = c < K ? *(const uint4*)(x + c) : make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TOK; ++j) {
+            float acc[ROWS] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const unsigned xu[4] = {xr[j][i].x, xr[j][i].y, xr[j][i].z, xr[j][i].w};
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const unsigned u[4] = {wr[r][i].x, wr[r][i].y, wr[r][i].z, wr[r][i].w};
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        acc[r] += __uint_as_float(u[q] << 16) * __uint_as_float(xu[q] << 16) +
+                                  __uint_as_float(u[q] & 0xffff0000u) * __uint_as_float(xu[q] & 0xffff0000u);
+                }
+            }
+            if (sb + j < s1) {                                              // (wave-uniform)
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    float d = wave_sum(acc[r]);
+                    if (lane == 0 && r0 + r < rows) {
+                        if (RELU_SQ) {
+                            d = fmaxf(d, 0.f);
+                            d *= d;
+                        }
+                        out[(size_t)(sb + j) * rows + r0 + r] = f2bf(d);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---- expert-sorted form (many tokens): the products are the vendor's, per expert over contiguous runs of sorted slots; these
 // kernels do the permutation in, the activation, and the weighted permutation out -----------------------------------------------
 template <typename T>
@@ -240,6 +308,30 @@ extern "C" int qsv_gather_rows(void* out, const void* src, const int64_t* order,
                  hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(n_rows), dim3(NT), 0, (hipStream_t)stream, (T*)out, (const T*)src,
                                     order, div, width));
     return qsv_launch_status("qsv_gather_rows");
+}
+// out[s, r] = act(W[e][r, :] . X[x_index ? x_index[s] / div : s, :]) for the sorted slots s in [offsets[e], offsets[e + 1]) of every
+// expert e; W [E, rows, K] bfloat16, act = relu^2 or nothing.  K % 8 == 0, K <= 4096.
+extern "C" int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
+                               int n_experts, int rows, int K, int relu_sq, void* stream) {
+    QSV_REQUIRE(out && X && W && offsets && n_experts > 0 && rows > 0 && div > 0, "qsv_expert_rows: bad arguments");
+    QSV_REQUIRE(K > 0 && K % 8 == 0 && K <= 4096, "qsv_expert_rows: inner width %d (a multiple of 8, at most 4096)", K);
+    QSV_REQUIRE(n_experts <= 65535, "qsv_expert_rows: too many experts");
+    const dim3 grid((rows + NW * ROWS - 1) / (NW * ROWS), n_experts), block(NT);
+#define QSV_ER(KI)                                                                                                           \
+    do {                                                                                                                     \
+        if (relu_sq)                                                                                                         \
+            hipLaunchKernelGGL((expert_rows_kernel<KI, true>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, \
+                               x_index, div, (const bf16_t*)W, offsets, rows, K);                                            \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((expert_rows_kernel<KI, false>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, \
+                               x_index, div, (const bf16_t*)W, offsets, rows, K);                                            \
+    } while (0)
+    if (K <= 512) QSV_ER(1);
+    else if (K <= 1024) QSV_ER(2);
+    else if (K <= 2048) QSV_ER(4);
+    else QSV_ER(8);
+#undef QSV_ER
+    return qsv_launch_status("qsv_expert_rows");
 }
 extern "C" int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream) {
     QSV_REQUIRE(a && n >= 0 && n < (1ll << 31) * NT, "qsv_relu_sq: bad arguments");

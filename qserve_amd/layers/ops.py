@@ -144,6 +144,9 @@ class HipOps:
         """up [E, ff, D], down [E, D, ff]; y[t] = sum_k wt[t, k] * down[idx[t, k]] relu(up[idx[t, k]] h[t])^2."""
         T, D = h.shape
         top_k, ff = idx.size(1), up.size(1)
+        if (self.code == BF16 and self.moe_token_slots < T * top_k <= self.moe_expert_major_slots and D % 8 == 0 and ff % 8 == 0
+                and D <= 4096 and ff <= 4096):
+            return self._moe_experts_expert_major(h, up, down, idx, wt)
         if T * top_k > self.moe_sorted_above:
             return self._moe_experts_sorted(h, up, down, idx, wt)
         act = torch.empty((T, top_k, ff), dtype=self.dtype, device=h.device)
@@ -160,6 +163,32 @@ class HipOps:
     # More (token, expert) slots than this: sort the slots by expert and run each expert as one matrix product.  Below it the
     # per-token kernels above are used: no host synchronisation, a fixed launch sequence.
     moe_sorted_above = 64
+
+    # (token, expert) slots: up to moe_token_slots the per-token kernels (two launches); up to moe_expert_major_slots the
+    # expert-major kernels (bfloat16; every expert weight read once, no host synchronisation); above, the expert-sorted vendor
+    # products (compute-bound sizes)
+    moe_token_slots = 8
+    moe_expert_major_slots = 1024
+
+    def _moe_experts_expert_major(self, h, up, down, idx, wt):
+        T, D = h.shape
+        E, ff, K = up.size(0), up.size(1), idx.size(1)
+        n = T * K
+        expert, order = torch.sort(idx.reshape(-1).long(), stable=True)   # order: sorted slot -> slot (t K + k)
+        # first sorted slot of every expert (and the end): a search in the sorted list - no count has to reach the host
+        offsets = torch.searchsorted(expert, torch.arange(E + 1, device=h.device))
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(n, device=h.device)                  # slot -> sorted slot
+        act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
+        ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
+        self.check(self.L.qsv_expert_rows(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), offsets.data_ptr(),
+                                          E, ff, D, 1, self._s()), "expert_rows(up)")
+        self.check(self.L.qsv_expert_rows(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), offsets.data_ptr(), E, D, ff, 0,
+                                          self._s()), "expert_rows(down)")
+        y = torch.empty((T, D), dtype=self.dtype, device=h.device)
+        self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
+                                          self._s()), "moe_combine")
+        return y
 
     def _moe_experts_sorted(self, h, up, down, idx, wt):
         T, D = h.shape

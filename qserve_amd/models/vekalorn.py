@@ -27,6 +27,16 @@ class Vekalorn:
         self.ops, self.width, self.vocab, self.eps = ops, width, vocab, eps
         self.embed, self.head, self.final_norm, self.layers = embed, head, final_norm, layers
         self.cache_rows = [L["mixer"].row_width for L in layers]
+        self.rotaries = list({id(L["mixer"].rotary): L["mixer"].rotary for L in layers if L["mixer"].rotary is not None}.values())
+
+    def reserve_positions(self, n):
+        """Make every rotary table cover positions [0, n)."""
+        for r in self.rotaries:
+            r.reserve(n)
+
+    def graph_signature(self):
+        """What a captured step holds by address and must find unchanged at replay."""
+        return tuple(r.table.data_ptr() for r in self.rotaries)
 
     @classmethod
     def from_config(cls, config, weights, ops, device, dtype, page=64):

@@ -76,7 +76,7 @@ class OpTimer:
              "moe_route", "moe_experts")
 
     def __init__(self, ops):
-        self.ops, self.events, self.on = ops, [], False
+        self.ops, self.events, self.calls, self.on = ops, [], [], False
         for n in self.NAMES:
             setattr(ops, n, self._wrap(n, getattr(ops, n)))
 
@@ -89,12 +89,30 @@ class OpTimer:
             r = fn(*a, **k)
             e1.record()
             self.events.append((name, e0, e1))
+            self.calls.append((name, fn, a, k))
             return r
         return timed
 
+    def replay(self, name, reps=20):
+        """The launches of `name` recorded in the last step(), each repeated back to back on the same arguments: ms per launch
+        without the host's share (what the kernel itself takes), summed over the step's launches."""
+        total = 0.0
+        for n, fn, a, k in self.calls:
+            if n != name:
+                continue
+            fn(*a, **k)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn(*a, **k)
+            e1.record()
+            torch.cuda.synchronize()
+            total += e0.elapsed_time(e1) / reps
+        return total
+
     def step(self, fn):
         """Run fn() with timing on -> ({op: ms summed over its launches}, total ms between first and last event)."""
-        self.events, self.on = [], True
+        self.events, self.calls, self.on = [], [], True
         t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0.record()
         fn()
@@ -123,7 +141,7 @@ def bench_vekalorn(name, s, dev, steps, warmup):
     from .engine import Engine
     cfg = vekalorn_config(s)
     NB, L, BP = 64, 1024, 8
-    eng = Engine(Vekalorn, cfg, random_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 256), max_seqs=NB)
+    eng = Engine(Vekalorn, cfg, random_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 384), max_seqs=NB)
     timer = OpTimer(eng.ops)
     g = torch.Generator().manual_seed(1)
     prompts = [torch.randint(0, VOCAB, (L,), generator=g).tolist() for _ in range(NB)]
@@ -135,6 +153,7 @@ def bench_vekalorn(name, s, dev, steps, warmup):
         want = [k * L + L - 1 for k in range(BP)]
         if i == BP:                                          # one step with events around every launch
             ops_pre, _ = timer.step(lambda: eng.execute(items, want))
+            att_pre_ms = timer.replay("latent_attention", 5)
             continue
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -151,12 +170,22 @@ def bench_vekalorn(name, s, dev, steps, warmup):
         eng.execute([(slots[j], nxt[j]) for j in range(NB)], want)
 
     res = {}
-    for label, above in (("sorted_experts", 0), ("per_token_experts", 10 ** 9)):
-        eng.ops.moe_sorted_above = above
-        res[label] = timed(decode, steps, warmup)
-    del eng.ops.moe_sorted_above
-    dec = timed(decode, steps, warmup)
+    forms = {"per_token": dict(moe_token_slots=10 ** 9, moe_sorted_above=10 ** 9),
+             "expert_major": dict(moe_token_slots=0, moe_expert_major_slots=10 ** 9),
+             "expert_sorted_vendor_products": dict(moe_token_slots=10 ** 9, moe_expert_major_slots=0, moe_sorted_above=0)}
+    for label, knobs in forms.items():
+        for k, v in knobs.items():
+            setattr(eng.ops, k, v)
+        res[label] = timed(decode, max(4, steps // 4), 2)
+        for k in knobs:
+            delattr(eng.ops, k)
+    dec_eager = timed(decode, steps, warmup)
     ops_dec, dec_events_ms = timer.step(decode)
+    att_dec_ms = timer.replay("latent_attention", 20)
+    moe_dec_ms = timer.replay("moe_experts", 20)
+    eng.decode_graphs = True                                 # the same steps replayed from a hipGraph
+    dec = timed(decode, steps, warmup)
+    graph_ok = any(v is not False for v in eng._graphs.values()) and bool(eng._graphs)
     ctx = eng.cache.length[slots[0]]
     # rooflines
     m1 = cfg["layers"][1]["mixer"]
@@ -166,16 +195,18 @@ def bench_vekalorn(name, s, dev, steps, warmup):
     T = BP * L
     flops = sum(sum(min(p + 1, s["window"]) if k == "latent_attention" else p + 1 for p in range(L)) * BP * H * (rows[k] + rank) * 2.0
                 for k in kinds)
-    att_pre = flops / (ops_pre["latent_attention"] * 1e-3) / 1e12
+    att_pre = flops / (att_pre_ms * 1e-3) / 1e12
     by = sum(NB * (min(ctx, s["window"]) if k == "latent_attention" else ctx) * rows[k] * 2.0 for k in kinds)
-    att_dec = by / (ops_dec["latent_attention"] * 1e-3) / 1e9
+    att_dec = by / (att_dec_ms * 1e-3) / 1e9
     moe_flops = LAYERS * T * s["top"] * 2 * 2.0 * s["ff"] * s["width"]
     moe_pre = moe_flops / (ops_pre["moe_experts"] * 1e-3) / 1e12
     moe_bytes = LAYERS * min(s["experts"], NB * s["top"]) * 2 * s["ff"] * s["width"] * 2.0
-    moe_dec = moe_bytes / (ops_dec["moe_experts"] * 1e-3) / 1e9
+    moe_dec = moe_bytes / (moe_dec_ms * 1e-3) / 1e9
     out = dict(model=f"Vekalorn-{name}", prefill_tokens_per_s=T / pre * 1e3, prefill_ms=pre, decode_tokens_per_s=NB / dec * 1e3,
-               decode_ms=dec, decode_ms_by_expert_form=res, decode_ms_gpu_events=dec_events_ms, context=ctx,
-               prefill_ops_ms=ops_pre, decode_ops_ms=ops_dec,
+               decode_ms=dec, decode_from_hipgraph=graph_ok, decode_ms_eager=dec_eager, decode_ms_eager_by_expert_form=res,
+               decode_ms_gpu_events=dec_events_ms, decode_experts_kernels_ms=moe_dec_ms, context=ctx,
+               prefill_ops_ms=ops_pre, decode_ops_ms=ops_dec, prefill_attention_kernels_ms=att_pre_ms,
+               decode_attention_kernels_ms=att_dec_ms,
                roofline=dict(prefill_attention_tflops=att_pre, prefill_attention_frac_bf16_peak=att_pre / BF16_PEAK_TFLOPS,
                              decode_attention_gbs=att_dec, decode_attention_frac_hbm=att_dec / HBM_PEAK_GBS,
                              prefill_experts_tflops=moe_pre, prefill_experts_frac_bf16_peak=moe_pre / BF16_PEAK_TFLOPS,

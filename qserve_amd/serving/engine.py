@@ -46,7 +46,9 @@ class StepBatch:
 
 class Engine:
     def __init__(self, model_cls, config, weights, dtype="bfloat16", device="cuda:0", max_tokens=4096, max_seqs=4,
-                 backend="hip", max_batch_tokens=2048, prefill_chunk=512, page=64):
+                 backend="hip", max_batch_tokens=2048, prefill_chunk=512, page=64, decode_graphs=False):
+        """decode_graphs: replay steps in which every sequence brings exactly one token from a hipGraph (captured per batch
+        size and context bucket; the launch sequence of such a step has no host synchronisation).  Off unless asked for."""
         self.dtype = DTYPES[dtype] if isinstance(dtype, str) else dtype
         self.device = torch.device(device)
         if self.dtype == torch.float32 and self.device.type == "cuda":
@@ -59,6 +61,8 @@ class Engine:
         self.scheduler = Scheduler(self.cache, max_batch_tokens, prefill_chunk)
         self.requests = {}
         self._ids = itertools.count()
+        self.decode_graphs = bool(decode_graphs) and backend == "hip"
+        self._graphs = {}                      # key -> _DecodeGraph, or False where capture failed (that shape runs eagerly)
 
     @classmethod
     def from_pretrained(cls, model_dir, **kw):
@@ -95,6 +99,10 @@ class Engine:
             pos += range(start, start + len(t))
         if not toks:
             return None
+        if self.decode_graphs and all(n == 1 for _, _, n in runs):
+            out = self._execute_graph(toks, seq, pos, rows, runs)
+            if out is not None:
+                return out[torch.tensor(list(want), dtype=torch.int64, device=self.device)] if want else None
         dev = self.device
         # (one host tensor, one copy: int64 rows and int32 metadata share a buffer)
         meta = torch.tensor([toks, seq, pos], dtype=torch.int32).to(dev)
@@ -104,6 +112,57 @@ class Engine:
         if not want:
             return None
         return self.model.logits(x, torch.tensor(list(want), dtype=torch.int32).to(dev))
+
+    # ---- decode steps from a hipGraph ------------------------------------------------------------------------------------------
+    GRAPH_BUCKET = 128                         # positions per context bucket (a graph freezes what is derived from max_pos)
+
+    def _execute_graph(self, toks, seq, pos, rows, runs):
+        """One token per sequence: fill the static inputs of the graph captured for (batch size, context bucket, model
+        signature) and replay it.  -> float logits for every row, or None if this shape runs eagerly."""
+        B, dev = len(toks), self.device
+        bucket = max(pos) // self.GRAPH_BUCKET
+        sig = self.model.graph_signature() if hasattr(self.model, "graph_signature") else ()
+        key = (B, bucket, sig)
+        G = self._graphs.get(key)
+        if G is False:
+            return None
+        meta = torch.tensor([toks, seq, pos], dtype=torch.int32)
+        slot = torch.tensor(rows, dtype=torch.int64)
+        if G is None:
+            if len(self._graphs) >= 16:
+                self._graphs.clear()
+            batch = StepBatch(tokens=None, seq=None, pos=None, slot=slot.to(dev), block_table=self.cache.block_table(),
+                              max_pos=(bucket + 1) * self.GRAPH_BUCKET - 1, n_tokens=B, items=list(runs))
+            m = meta.to(dev)
+            batch.tokens, batch.seq, batch.pos = m[0], m[1], m[2]
+            G = {"meta": m, "batch": batch, "rows": torch.arange(B, dtype=torch.int32, device=dev)}
+            if hasattr(self.model, "reserve_positions"):
+                self.model.reserve_positions(batch.max_pos + 1)
+                key = (B, bucket, self.model.graph_signature() if hasattr(self.model, "graph_signature") else ())
+            try:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):                      # warm-up outside capture (allocator, lazy initialisation)
+                    self.model.logits(self.model.forward(batch, self.cache.pools), G["rows"])
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    G["logits"] = self.model.logits(self.model.forward(batch, self.cache.pools), G["rows"])
+                G["graph"] = g
+            except Exception:                                      # e.g. a launch sequence that synchronises: run eagerly
+                torch.cuda.synchronize()
+                self._graphs[key] = False
+                return None
+            self._graphs[key] = G
+        batch = G["batch"]
+        G["meta"].copy_(meta)
+        batch.slot.copy_(slot)
+        for tpb, t in batch._tiles.items():
+            t.copy_(torch.tensor([(s, first, 1) for s, first, _ in runs], dtype=torch.int32).reshape(-1, 3))
+        self.cache.block_table()
+        G["graph"].replay()
+        return G["logits"]
 
     # ---- generation ------------------------------------------------------------------------------------------------------------
     def add_request(self, prompt, params=None, request_id=None):
