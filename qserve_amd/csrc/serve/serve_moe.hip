@@ -9,8 +9,35 @@ constexpr int NT = 256;
 constexpr int NW = NT / 64;
 constexpr int MAX_EXPERTS = 1024;
 
-// One workgroup per token.  z = router . h by the waves, then one thread does the selection (at most a few thousand steps).
-// Ties go to the lower index, for groups and for experts.
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 u = *(const uint4*)p;
+    const unsigned w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+// (value, index) of the largest value over a wave; ties go to the lower index.  Lanes without a candidate pass index -1.
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, 64);
+        const int oi = __shfl_xor(i, o, 64);
+        if (oi >= 0 && (i < 0 || ov > v || (ov == v && oi < i))) {
+            v = ov;
+            i = oi;
+        }
+    }
+}
+
+// One workgroup per token.  z = router . h by the four waves (16-byte loads where the width allows), then wave 0 selects:
+// softmax, group maxima, the best groups and the top experts by repeated wave-wide argmax.  Ties go to the lower index, for
+// groups and for experts.
 template <typename T>
 __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx, float* __restrict__ weight,
                                                        const T* __restrict__ h, const T* __restrict__ router, int D, int E,
@@ -24,42 +51,82 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
     for (int e = w; e < E; e += NW) {
         const T* r = router + (size_t)e * D;
         float d = 0.f;
-        for (int i = lane; i < D; i += 64) d += ld(r, i) * ld(x, i);
+        if (D % 8 == 0) {
+            for (int c = lane * 8; c < D; c += 64 * 8) {
+                float a[8], b[8];
+                load8(r + c, a);
+                load8(x + c, b);
+#pragma unroll
+                for (int q = 0; q < 8; ++q) d += a[q] * b[q];
+            }
+        } else {
+            for (int i = lane; i < D; i += 64) d += ld(r, i) * ld(x, i);
+        }
         d = wave_sum(d);
         if (lane == 0) s[e] = d;
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    float mx = s[0];
-    for (int e = 1; e < E; ++e) mx = fmaxf(mx, s[e]);
-    float sum = 0.f;
-    for (int e = 0; e < E; ++e) {
-        s[e] = expf(s[e] - mx);
-        sum += s[e];
+    // (the other three waves only keep the barriers company from here on: the selection is a few hundred steps of one wave)
+    const bool sel = w == 0;
+    float inv = 0.f;
+    if (sel) {                                              // softmax over all experts
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float p = expf(s[e] - mx);
+            s[e] = p;
+            sum += p;
+        }
+        inv = 1.0f / wave_sum(sum);
+        for (int e = lane; e < E; e += 64) {
+            s[e] *= inv;
+            ok[e] = 0;
+        }
     }
-    const float inv = 1.0f / sum;
-    for (int e = 0; e < E; ++e) s[e] *= inv;
+    __syncthreads();
     const int per = E / G;
-    for (int g = 0; g < G; ++g) {
-        float v = s[g * per];
-        for (int e = 1; e < per; ++e) v = fmaxf(v, s[g * per + e]);
-        gs[g] = v;
+    if (sel) {                                              // group maxima
+        for (int g = lane; g < G; g += 64) {
+            float v = s[g * per];
+            for (int e = 1; e < per; ++e) v = fmaxf(v, s[g * per + e]);
+            gs[g] = v;
+        }
     }
-    for (int e = 0; e < E; ++e) ok[e] = 0;
-    for (int k = 0; k < keep; ++k) {
-        int best = -1;
-        for (int g = 0; g < G; ++g)
-            if (gs[g] >= 0.f && (best < 0 || gs[g] > gs[best])) best = g;
-        gs[best] = -1.f;                            // scores are probabilities: -1 marks a taken group
-        for (int e = 0; e < per; ++e) ok[best * per + e] = 1;
+    __syncthreads();
+    for (int k = 0; k < keep; ++k) {                        // the `keep` best groups
+        if (sel) {
+            float bv = 0.f;
+            int bi = -1;
+            for (int g = lane; g < G; g += 64)
+                if (gs[g] >= 0.f && (bi < 0 || gs[g] > bv)) {
+                    bv = gs[g];
+                    bi = g;
+                }
+            wave_argmax(bv, bi);
+            if (lane == 0) gs[bi] = -1.f;                   // scores are probabilities: -1 marks a taken group
+            for (int e = lane; e < per; e += 64) ok[bi * per + e] = 1;
+        }
+        __syncthreads();
     }
-    for (int k = 0; k < top_k; ++k) {
-        int best = -1;
-        for (int e = 0; e < E; ++e)
-            if (ok[e] && (best < 0 || s[e] > s[best])) best = e;
-        ok[best] = 0;
-        idx[t * top_k + k] = best;
-        weight[t * top_k + k] = s[best];
+    for (int k = 0; k < top_k; ++k) {                       // the top_k eligible experts
+        if (sel) {
+            float bv = 0.f;
+            int bi = -1;
+            for (int e = lane; e < E; e += 64)
+                if (ok[e] && (bi < 0 || s[e] > bv)) {
+                    bv = s[e];
+                    bi = e;
+                }
+            wave_argmax(bv, bi);
+            if (lane == 0) {
+                ok[bi] = 0;
+                idx[t * top_k + k] = bi;
+                weight[t * top_k + k] = bv;
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -110,19 +177,6 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(T* __restrict__ y, const T
 
 // The same two kernels for widths that are multiples of 8: 16-byte weight loads and four output rows per wave in flight at once
 // (the scalar forms above wait for one row's loads before they issue the next row's: latency-bound at real layer sizes).
-__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
-    const uint4 u = *(const uint4*)p;
-    const unsigned w[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        v[2 * i] = __uint_as_float(w[i] << 16);
-        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-    }
-}
-__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
-    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
 constexpr int ROWS = 4;      // output rows a wave works on at once
 
 template <typename T>

@@ -1,6 +1,6 @@
 """Command line of the serving engine.
 
-    python -m qserve_amd.serving generate --model DIR --prompt 1,2,3 [--prompt ...] [--max-new N] [--dtype ...]
+    python -m qserve_amd.serving generate --model DIR --prompt 1,2,3 [--prompt ...] [--max-new N] [--dtype ...] [--graphs]
     python -m qserve_amd.serving trace    --model DIR --dtype ... --out DIR --max-tokens N     (steps on standard input)
     python -m qserve_amd.serving models
 """
@@ -37,9 +37,11 @@ def main():
     ap.add_argument("--max-tokens", type=int, default=8192)
     ap.add_argument("--max-seqs", type=int, default=4)
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--graphs", action="store_true", help="replay single-token steps from hipGraphs")
     a = ap.parse_args(argv)
     from . import Engine, SamplingParams
-    eng = Engine.from_pretrained(a.model, dtype=a.dtype, device=a.device, max_tokens=a.max_tokens, max_seqs=a.max_seqs)
+    eng = Engine.from_pretrained(a.model, dtype=a.dtype, device=a.device, max_tokens=a.max_tokens, max_seqs=a.max_seqs,
+                                 decode_graphs=a.graphs)
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in a.prompt]
     outs = eng.generate(prompts, SamplingParams(max_new=a.max_new, temperature=a.temperature, top_k=a.top_k, top_p=a.top_p,
                                                 seed=a.seed))

@@ -113,7 +113,7 @@ def assert_close(got, ref, tol, what=""):
     assert err <= tol * scale, f"{what}: max error {err:.3e} (allowed {tol * scale:.3e})"
 
 
-F32_TOL = 3e-5
+F32_TOL = 1e-4      # whole-model float32 runs against float64: rounding through four layers and their norms (a fault shows at 1e-2 and above)
 
 
 # ---- mechanisms alone -------------------------------------------------------------------------------------------------------------
