@@ -112,8 +112,9 @@ int launch_wave(void* out, const float* qf, const void* pool, const int32_t* bt,
     else if (R <= 256) QSV_ATT(4);
     else if (R <= 384) QSV_ATT(6);
     else if (R <= 576) QSV_ATT(9);
+    else if (R <= 1024) QSV_ATT(16);
     else {
-        qsv_set_error("qsv_latent_attention: cache rows of %d elements (at most 576)", R);
+        qsv_set_error("qsv_latent_attention: cache rows of %d elements (at most 1024)", R);
         return QSV_EINVAL;
     }
 #undef QSV_ATT

@@ -259,6 +259,7 @@ __global__ __launch_bounds__(NT) void moe_down_vec_kernel(T* __restrict__ y, con
 // ---- expert-major form (decoding and short portions, bfloat16): slots sorted by expert ON THE DEVICE, workgroup = (16 output rows,
 // expert); a wave keeps its four weight rows in registers (packed bfloat16) and walks the tokens routed to the expert, so every
 // weight is read once per step however many tokens share the expert.  No host synchronisation. ----------------------------------
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
 template <int KI, bool RELU_SQ>
 __global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
                                                          const int64_t* __restrict__ x_index, int div, const bf16_t* __restrict__ W,
@@ -302,9 +303,8 @@ __global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ ou
                 for (int r = 0; r < ROWS; ++r) {
                     const unsigned u[4] = {wr[r][i].x, wr[r][i].y, wr[r][i].z, wr[r][i].w};
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        acc[r] += __uint_as_float(u[q] << 16) * __uint_as_float(xu[q] << 16) +
-                                  __uint_as_float(u[q] & 0xffff0000u) * __uint_as_float(xu[q] & 0xffff0000u);
+                    for (int q = 0; q < 4; ++q)                           // v_dot2_f32_bf16: two products per instruction, no unpacking
+                        acc[r] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, u[q]), __builtin_bit_cast(bf2, xu[q]), acc[r], false);
                 }
             }
             if (sb + j < s1) {                                              // (wave-uniform)
