@@ -27,7 +27,7 @@ __device__ __forceinline__ unsigned pack_bf2(float a, float b) { return (unsigne
 
 // RT: 32-element steps along a cache row (R <= 32 RT); CT: 16-column tiles of the output (rank <= 16 CT).
 template <int RT, int CT>
-__global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
+__global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ qf, const bf16_t* __restrict__ pool,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ pos, const int32_t* __restrict__ tiles,
     int window, int H, int rank, int R, int page, int HP, int TQ, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     // ---- merge the key splits (waves grp + G s, s = 1 .. S - 1, into wave grp) ----
     if (S > 1) {                                         // (block-uniform)
         __syncthreads();                                 // the last tile has been read: LDS becomes scratch
-        float* ml = scratch + NWV * 64 * 4;              // [NWV][64][2]
+        float* ml = scratch + NWV * 8 * 64 * 4;          // [NWV][64][2], behind the accumulator exchange area
         if (active && sp > 0) {
             ml[(w * 64 + lane) * 2] = m;
             ml[(w * 64 + lane) * 2 + 1] = l;
@@ -207,15 +207,25 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
             l = L;
             m = M;                                       // (what a cross-workgroup merge reads)
         }
+        // accumulators through LDS, MB column tiles per exchange (two barriers each)
+        constexpr int MB = CT < 8 ? CT : 8;
 #pragma unroll
-        for (int c = 0; c < CT; ++c) {
+        for (int c0 = 0; c0 < CT; c0 += MB) {
             __syncthreads();
-            if (active && sp > 0) *(v4f*)(scratch + (w * 64 + lane) * 4) = oacc[c];
+            if (active && sp > 0) {
+#pragma unroll
+                for (int j = 0; j < MB; ++j)
+                    if (c0 + j < CT) *(v4f*)(scratch + ((w * MB + j) * 64 + lane) * 4) = oacc[c0 + j];
+            }
             __syncthreads();
             if (active && sp == 0) {
-                v4f a = oacc[c] * f[0];
-                for (int s = 1; s < S; ++s) a += *(const v4f*)(scratch + ((grp + G * s) * 64 + lane) * 4) * f[s];
-                oacc[c] = a;
+#pragma unroll
+                for (int j = 0; j < MB; ++j)
+                    if (c0 + j < CT) {
+                        v4f a = oacc[c0 + j] * f[0];
+                        for (int s = 1; s < S; ++s) a += *(const v4f*)(scratch + (((grp + G * s) * MB + j) * 64 + lane) * 4) * f[s];
+                        oacc[c0 + j] = a;
+                    }
             }
         }
     }
@@ -303,7 +313,7 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
 #define QSV_MFMA(RT, CT)                                                                                                     \
     do {                                                                                                                     \
         size_t lds = (size_t)(BN * (32 * RT + 8) + 16 * CT * VS) * 2;                                                        \
-        const size_t need = (size_t)NWV * 64 * 6 * 4;                                                                       \
+        const size_t need = (size_t)NWV * 64 * (8 * 4 + 2) * 4;       /* merge scratch */                                                                       \
         if (lds < need) lds = need;                                                                                          \
         if (lds > 64 * 1024) {   /* above the default limit of dynamic LDS: raise it for this kernel */                        \
             const hipError_t e = hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<RT, CT>,                      \
