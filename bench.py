@@ -84,7 +84,7 @@ def parse():
     ap.add_argument("--design", default=None, choices=["vekalorn"],
                     help="instead of the default workload: prompt-phase and decode throughput of a design served by the paged "
                          "engine (qserve_amd/serving) beside the W4A8KV4 Llama engine at equal size; one JSON line per size")
-    ap.add_argument("--design-sizes", default="w2048,w4096", help="with --design: comma-separated size names (qserve_amd/serving/bench.py)")
+    ap.add_argument("--design-sizes", default="w2048,w2048r256,w4096", help="with --design: comma-separated size names (qserve_amd/serving/bench.py)")
     a = ap.parse_args()
     preset = CONFIGS[a.config] if a.config else CONFIGS[2]
     for k, v in preset.items():

@@ -94,6 +94,10 @@ int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx,
  * weight is read once per launch.  K a multiple of 8, at most 4096. */
 int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
                     int n_experts, int rows, int K, int relu_sq, void* stream);
+/* Grouped expert product on the bf16 matrix cores (prompt phase): the same out[s, n] for work tiles (expert, first sorted slot,
+ * slots <= 64) listed in tiles int32 [n_tiles, 3]; K a multiple of 32, n_rows a multiple of 4, n_tiles <= 65535. */
+int qsv_grouped_gemm(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int32_t* tiles,
+                     int n_tiles, int n_rows, int K, int relu_sq, void* stream);
 int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, int n_rows, int width, int dtype, void* stream);
 int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream);
 int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n_tokens, int top_k, int width,

@@ -163,6 +163,8 @@ class HipOps:
     # More (token, expert) slots than this: sort the slots by expert and run each expert as one matrix product.  Below it the
     # per-token kernels above are used: no host synchronisation, a fixed launch sequence.
     moe_sorted_above = 64
+    # the sorted form's products: the grouped matrix-core kernel (bfloat16, widths multiples of 32) or one vendor product per expert
+    moe_grouped_kernel = True
 
     # (token, expert) slots: up to moe_token_slots the per-token kernels (two launches); up to moe_expert_major_slots the
     # expert-major kernels (bfloat16; every expert weight read once, no host synchronisation); above, the expert-sorted vendor
@@ -199,6 +201,24 @@ class HipOps:
         counts = torch.bincount(flat, minlength=E).tolist()            # (host synchronisation: the runs' lengths)
         inv = torch.empty_like(order)
         inv[order] = torch.arange(n, device=h.device)                  # slot -> sorted slot
+        if self.moe_grouped_kernel and self.code == BF16 and D % 32 == 0 and ff % 32 == 0:
+            # own grouped matrix-core kernel: gather in its loads, relu^2 in the first product's epilogue
+            tiles, a = [], 0
+            for e, c in enumerate(counts):
+                tiles += [(e, a + o, min(64, c - o)) for o in range(0, c, 64)]
+                a += c
+            act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
+            ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
+            for lo in range(0, len(tiles), 65535):
+                tl = torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device)
+                self.check(self.L.qsv_grouped_gemm(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), tl.data_ptr(),
+                                                   tl.size(0), ff, D, 1, self._s()), "grouped_gemm(up)")
+                self.check(self.L.qsv_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), tl.data_ptr(),
+                                                   tl.size(0), D, ff, 0, self._s()), "grouped_gemm(down)")
+            y = torch.empty((T, D), dtype=self.dtype, device=h.device)
+            self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
+                                              self._s()), "moe_combine")
+            return y
         xs = torch.empty((n, D), dtype=self.dtype, device=h.device)
         self.check(self.L.qsv_gather_rows(xs.data_ptr(), h.data_ptr(), order.data_ptr(), K, n, D, self.code, self._s()),
                    "gather_rows")

@@ -593,10 +593,11 @@ def test_matrix_core_attention_matches_the_wave_kernel(heads, rank, rot):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("E,top,ff,D,T", [(6, 3, 24, 40, 33), (16, 4, 136, 264, 64), (4, 2, 8, 520, 5), (8, 8, 1032, 2056, 3)])
+@pytest.mark.parametrize("E,top,ff,D,T", [(6, 3, 24, 40, 33), (16, 4, 136, 264, 64), (4, 2, 8, 520, 5), (8, 8, 1032, 2056, 3),
+                                          (8, 2, 96, 160, 200), (3, 1, 32, 32, 70), (4, 4, 1408, 1024, 150)])
 def test_expert_forms_agree_in_bfloat16(E, top, ff, D, T):
-    """Per-token kernels, expert-major kernels and expert-sorted vendor products on the same bfloat16 inputs, against the
-    float64 sum over the chosen experts."""
+    """Per-token kernels, expert-major kernels, the grouped matrix-core kernel (widths that are multiples of 32) and
+    expert-sorted vendor products on the same bfloat16 inputs, against the float64 sum over the chosen experts."""
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     dev = "cuda:0"
@@ -617,7 +618,9 @@ def test_expert_forms_agree_in_bfloat16(E, top, ff, D, T):
             ref[t] += wt[t, k].double() * (down[e].double() @ a)
     forms = {"per-token": dict(moe_token_slots=10 ** 9, moe_sorted_above=10 ** 9),
              "expert-major": dict(moe_token_slots=0, moe_expert_major_slots=10 ** 9),
-             "expert-sorted": dict(moe_token_slots=10 ** 9, moe_expert_major_slots=0, moe_sorted_above=0)}
+             "expert-sorted, grouped kernel": dict(moe_token_slots=10 ** 9, moe_expert_major_slots=0, moe_sorted_above=0),
+             "expert-sorted, vendor products": dict(moe_token_slots=10 ** 9, moe_expert_major_slots=0, moe_sorted_above=0,
+                                                    moe_grouped_kernel=False)}
     for name, knobs in forms.items():
         o = make_ops("hip", torch.bfloat16, dev)
         for k, v in knobs.items():
