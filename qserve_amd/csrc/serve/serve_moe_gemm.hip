@@ -1,11 +1,11 @@
 // serve_moe_gemm.hip -- grouped expert products on the bf16 matrix cores for the prompt phase (many tokens per expert).
 //
-// The (token, expert) slots are sorted by expert; a work tile = up to 64 consecutive sorted slots of ONE expert (tile list made
-// by the host from the run lengths).  A workgroup computes 128 weight rows x 64 slots of out[s, n] = act(W[e][n, :] . x(s)):
+// The (token, expert) slots are sorted by expert; a work tile = up to 128 consecutive sorted slots of ONE expert (tile list made
+// by the host from the run lengths).  A workgroup computes 128 weight rows x 128 slots of out[s, n] = act(W[e][n, :] . x(s)):
 // both operands are contiguous along the reduction, so with the weight rows as the A operand and the slots' inputs as the B
 // operand (v_mfma_f32_16x16x32_bf16) a lane ends up with 4 consecutive n of one slot - an 8-byte store.  The input row of a
 // slot is fetched through an index (the gather into sorted order is part of the load), relu(.)^2 is the epilogue of the first
-// product.  K steps of 32 through LDS (stride 40 elements: conflict-free 16-byte reads), the next step's pieces in flight in
+// product.  K steps of 64 through LDS (stride 72 elements: conflict-free 16-byte reads), the next step's pieces in flight in
 // registers while this one is multiplied.
 #include "serve_common.h"
 
@@ -16,9 +16,11 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
 constexpr int BNW = 128;     // weight rows per workgroup (32 per wave)
-constexpr int BS = 64;       // slots per tile
-constexpr int KS = 32;       // reduction elements per step
+constexpr int BS = 128;      // slots per tile
+constexpr int KS = 64;       // reduction elements per step
 constexpr int LS = KS + 8;   // LDS row stride (elements)
+constexpr int CPR = KS / 8;  // 16-byte pieces per row and step
+constexpr int NPA = BNW * CPR / 256, NPB = BS * CPR / 256;   // pieces per thread
 
 __device__ __forceinline__ unsigned pack_bf2(float a, float b) { return (unsigned)f2bf(a) | ((unsigned)f2bf(b) << 16); }
 
@@ -33,59 +35,71 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(bf16_t* __restrict__ 
     const int col = lane & 15, g4 = lane >> 4;
     const int e = tiles[3 * blockIdx.y], s_first = tiles[3 * blockIdx.y + 1], ns = tiles[3 * blockIdx.y + 2];
     const int n0 = blockIdx.x * BNW;
-    // this thread's pieces of a K step: two of the weight tile (rows q / 4, 16-byte piece q % 4), one of the input tile
-    const bf16_t* ap[2];
-    bool aok[2];
+    // this thread's pieces of a K step: piece q = tid + 256 i is row q / CPR, 16 bytes number q % CPR
+    const bf16_t* ap[NPA];
+    const bf16_t* bp[NPB];
+    bool aok[NPA], bok[NPB];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int q = tid + 256 * i, row = q >> 2, cc = q & 3;
+    for (int i = 0; i < NPA; ++i) {
+        const int q = tid + 256 * i, row = q / CPR, cc = q % CPR;
         aok[i] = n0 + row < N;
         ap[i] = W + ((size_t)e * N + (aok[i] ? n0 + row : 0)) * (size_t)K + cc * 8;
     }
-    const int brow = tid >> 2, bcc = tid & 3;
-    const bool bok = brow < ns;
-    const int64_t s = s_first + (bok ? brow : 0);
-    const bf16_t* bp = X + (size_t)(x_index ? x_index[s] / div : s) * (size_t)K + bcc * 8;
-
-    v4f acc[2][4];
+#pragma unroll
+    for (int i = 0; i < NPB; ++i) {
+        const int q = tid + 256 * i, row = q / CPR, cc = q % CPR;
+        bok[i] = row < ns;
+        const int64_t s = s_first + (bok[i] ? row : 0);
+        bp[i] = X + (size_t)(x_index ? x_index[s] / div : s) * (size_t)K + cc * 8;
+    }
+    v4f acc[2][BS / 16];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int nt = 0; nt < BS / 16; ++nt) acc[mt][nt] = v4f{0.f, 0.f, 0.f, 0.f};
     const v4u zero = {0u, 0u, 0u, 0u};
-    v4u ra[2], rb;
-    ra[0] = aok[0] ? *(const v4u*)ap[0] : zero;
-    ra[1] = aok[1] ? *(const v4u*)ap[1] : zero;
-    rb = bok ? *(const v4u*)bp : zero;
+    v4u ra[NPA], rb[NPB];
+#pragma unroll
+    for (int i = 0; i < NPA; ++i) ra[i] = aok[i] ? *(const v4u*)ap[i] : zero;
+#pragma unroll
+    for (int i = 0; i < NPB; ++i) rb[i] = bok[i] ? *(const v4u*)bp[i] : zero;
     for (int k0 = 0; k0 < K; k0 += KS) {
         __syncthreads();                                            // the previous step has been read
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < NPA; ++i) {
             const int q = tid + 256 * i;
-            *(v4u*)(As + (q >> 2) * LS + (q & 3) * 8) = ra[i];
+            *(v4u*)(As + (q / CPR) * LS + (q % CPR) * 8) = ra[i];
         }
-        *(v4u*)(Bs + brow * LS + bcc * 8) = rb;
+#pragma unroll
+        for (int i = 0; i < NPB; ++i) {
+            const int q = tid + 256 * i;
+            *(v4u*)(Bs + (q / CPR) * LS + (q % CPR) * 8) = rb[i];
+        }
         __syncthreads();
         if (k0 + KS < K) {                                          // next step's pieces: in flight during the products
-            ra[0] = aok[0] ? *(const v4u*)(ap[0] + k0 + KS) : zero;
-            ra[1] = aok[1] ? *(const v4u*)(ap[1] + k0 + KS) : zero;
-            rb = bok ? *(const v4u*)(bp + k0 + KS) : zero;
+#pragma unroll
+            for (int i = 0; i < NPA; ++i) ra[i] = aok[i] ? *(const v4u*)(ap[i] + k0 + KS) : zero;
+#pragma unroll
+            for (int i = 0; i < NPB; ++i) rb[i] = bok[i] ? *(const v4u*)(bp[i] + k0 + KS) : zero;
         }
-        v4u a[2], b[4];
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) a[mt] = *(const v4u*)(As + (32 * w + 16 * mt + col) * LS + 8 * g4);
+        for (int kk = 0; kk < KS; kk += 32) {
+            v4u a[2];
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) b[nt] = *(const v4u*)(Bs + (16 * nt + col) * LS + 8 * g4);
+            for (int mt = 0; mt < 2; ++mt) a[mt] = *(const v4u*)(As + (32 * w + 16 * mt + col) * LS + kk + 8 * g4);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+            for (int nt = 0; nt < BS / 16; ++nt) {
+                const v4u b = *(const v4u*)(Bs + (16 * nt + col) * LS + kk + 8 * g4);
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a[mt]), __builtin_bit_cast(bf8, b[nt]),
-                                                                      acc[mt][nt], 0, 0, 0);
+                for (int mt = 0; mt < 2; ++mt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a[mt]), __builtin_bit_cast(bf8, b),
+                                                                          acc[mt][nt], 0, 0, 0);
+            }
+        }
     }
     // this lane: slot 16 nt + col, weight rows n0 + 32 w + 16 mt + 4 g4 + (0 .. 3)
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
+    for (int nt = 0; nt < BS / 16; ++nt) {
         const int sl = 16 * nt + col;
         if (sl >= ns) continue;
 #pragma unroll
@@ -107,12 +121,14 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(bf16_t* __restrict__ 
 }
 }  // namespace
 
-// out[s, n] = act(W[e][n, :] . X[x_index ? x_index[s] / div : s, :]) for every tile (e, first sorted slot, slots <= 64);
-// W [E, N, K], all bfloat16; K % 32 == 0, N % 4 == 0.
+// out[s, n] = act(W[e][n, :] . X[x_index ? x_index[s] / div : s, :]) for every tile (e, first sorted slot, slots <= qsv_grouped_gemm_tile_slots());
+// W [E, N, K], all bfloat16; K % 64 == 0, N % 4 == 0.
+extern "C" int qsv_grouped_gemm_tile_slots(void) { return BS; }
+extern "C" int qsv_grouped_gemm_k_step(void) { return KS; }
 extern "C" int qsv_grouped_gemm(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int32_t* tiles,
                                 int n_tiles, int N, int K, int relu_sq, void* stream) {
     QSV_REQUIRE(out && X && W && tiles && div > 0 && n_tiles >= 0, "qsv_grouped_gemm: bad arguments");
-    QSV_REQUIRE(N > 0 && N % 4 == 0 && K > 0 && K % KS == 0, "qsv_grouped_gemm: N %d (a multiple of 4), K %d (a multiple of 32)", N, K);
+    QSV_REQUIRE(N > 0 && N % 4 == 0 && K > 0 && K % KS == 0, "qsv_grouped_gemm: N %d (a multiple of 4), K %d (a multiple of 64)", N, K);
     QSV_REQUIRE(n_tiles <= 65535, "qsv_grouped_gemm: %d tiles (at most 65535 per launch)", n_tiles);
     if (n_tiles == 0) return QSV_OK;
     const dim3 grid((N + BNW - 1) / BNW, n_tiles), block(256);

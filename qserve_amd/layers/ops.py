@@ -163,7 +163,7 @@ class HipOps:
     # More (token, expert) slots than this: sort the slots by expert and run each expert as one matrix product.  Below it the
     # per-token kernels above are used: no host synchronisation, a fixed launch sequence.
     moe_sorted_above = 64
-    # the sorted form's products: the grouped matrix-core kernel (bfloat16, widths multiples of 32) or one vendor product per expert
+    # the sorted form's products: the grouped matrix-core kernel (bfloat16, widths multiples of its K step) or one vendor product per expert
     moe_grouped_kernel = True
 
     # (token, expert) slots: up to moe_token_slots the per-token kernels (two launches); up to moe_expert_major_slots the
@@ -201,11 +201,12 @@ class HipOps:
         counts = torch.bincount(flat, minlength=E).tolist()            # (host synchronisation: the runs' lengths)
         inv = torch.empty_like(order)
         inv[order] = torch.arange(n, device=h.device)                  # slot -> sorted slot
-        if self.moe_grouped_kernel and self.code == BF16 and D % 32 == 0 and ff % 32 == 0:
+        ks, ts = self.L.qsv_grouped_gemm_k_step(), self.L.qsv_grouped_gemm_tile_slots()
+        if self.moe_grouped_kernel and self.code == BF16 and D % ks == 0 and ff % ks == 0:
             # own grouped matrix-core kernel: gather in its loads, relu^2 in the first product's epilogue
             tiles, a = [], 0
             for e, c in enumerate(counts):
-                tiles += [(e, a + o, min(64, c - o)) for o in range(0, c, 64)]
+                tiles += [(e, a + o, min(ts, c - o)) for o in range(0, c, ts)]
                 a += c
             act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
             ys = torch.empty((n, D), dtype=self.dtype, device=h.device)

@@ -25,6 +25,8 @@ SIGNATURES = {
     "qsv_moe_route": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "qsv_moe_up": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "qsv_expert_rows": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "qsv_grouped_gemm_tile_slots": (_i, []),
+    "qsv_grouped_gemm_k_step": (_i, []),
     "qsv_grouped_gemm": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "qsv_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "qsv_relu_sq": (_i, [_vp, _i64, _i, _vp]),

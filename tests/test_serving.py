@@ -594,9 +594,9 @@ def test_matrix_core_attention_matches_the_wave_kernel(heads, rank, rot):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("E,top,ff,D,T", [(6, 3, 24, 40, 33), (16, 4, 136, 264, 64), (4, 2, 8, 520, 5), (8, 8, 1032, 2056, 3),
-                                          (8, 2, 96, 160, 200), (3, 1, 32, 32, 70), (4, 4, 1408, 1024, 150)])
+                                          (8, 2, 128, 192, 300), (3, 1, 64, 64, 70), (4, 4, 1408, 1024, 150)])
 def test_expert_forms_agree_in_bfloat16(E, top, ff, D, T):
-    """Per-token kernels, expert-major kernels, the grouped matrix-core kernel (widths that are multiples of 32) and
+    """Per-token kernels, expert-major kernels, the grouped matrix-core kernel (widths that are multiples of 64) and
     expert-sorted vendor products on the same bfloat16 inputs, against the float64 sum over the chosen experts."""
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
