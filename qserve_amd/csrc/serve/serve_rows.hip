@@ -155,29 +155,33 @@ extern "C" int qsv_latent_prep(const void* down, int64_t down_stride, int q_off,
 }
 
 // ---- the query in the latent space: [absorbed part | rotated part], scaled, float ---------------------------------------------
+// One workgroup per token, all heads: the absorbed part is a strided gather ([H, T, rank] -> [T, H, rank + rot]), the rotated
+// part a handful of values per head.
 template <typename T>
 __global__ __launch_bounds__(NT) void latent_query_kernel(float* __restrict__ qf, const T* __restrict__ q,
                                                           const T* __restrict__ q_abs, const float* __restrict__ rope,
                                                           const int32_t* __restrict__ pos, float scale, int n_tokens, int H,
                                                           int dim, int rot_dim, int rot_n, int rank) {
-    const size_t t = blockIdx.x / H;
-    const int h = blockIdx.x % H;
+    const size_t t = blockIdx.x;
     const int R = rank + rot_dim;
-    float* dst = qf + (t * H + h) * (size_t)R;
-    const T* qa = q_abs + ((size_t)h * n_tokens + t) * (size_t)rank;
-    for (int i = threadIdx.x; i < rank; i += NT) dst[i] = ld(qa, i) * scale;
-    const T* qr = q + (t * H + h) * (size_t)(dim + rot_dim) + dim;
+    float* dst = qf + t * H * (size_t)R;
+    for (int i = threadIdx.x; i < H * rank; i += NT) {
+        const int h = i / rank, c = i - h * rank;
+        dst[(size_t)h * R + c] = ld(q_abs, ((size_t)h * n_tokens + t) * (size_t)rank + c) * scale;
+    }
     const int half = rot_n / 2;
     const float* cs = rope ? rope + (size_t)pos[t] * (size_t)rot_n : nullptr;
-    for (int i = threadIdx.x; i < rot_dim; i += NT) {
-        float v = ld(qr, i);
-        if (i < rot_n) {
-            const int p = i >> 1;
-            const float c = cs[p], sn = cs[half + p];
+    for (int i = threadIdx.x; i < H * rot_dim; i += NT) {
+        const int h = i / rot_dim, c = i - h * rot_dim;
+        const T* qr = q + (t * H + h) * (size_t)(dim + rot_dim) + dim;
+        float v = ld(qr, c);
+        if (c < rot_n) {
+            const int p = c >> 1;
+            const float co = cs[p], sn = cs[half + p];
             const float u = ld(qr, 2 * p), w2 = ld(qr, 2 * p + 1);
-            v = (i & 1) ? (w2 * c + u * sn) : (u * c - w2 * sn);
+            v = (c & 1) ? (w2 * co + u * sn) : (u * co - w2 * sn);
         }
-        dst[rank + i] = v * scale;
+        dst[(size_t)h * R + rank + c] = v * scale;
     }
 }
 extern "C" int qsv_latent_query(float* qf, const void* q, const void* q_abs, const float* rope, const int32_t* pos, float scale,
@@ -188,7 +192,7 @@ extern "C" int qsv_latent_query(float* qf, const void* q, const void* q_abs, con
     if (n == 0) return QSV_OK;
     QSV_REQUIRE((int64_t)n * H < (1ll << 31), "qsv_latent_query: too many (token, head) pairs");
     QSV_DISPATCH(dtype, "qsv_latent_query",
-                 hipLaunchKernelGGL(latent_query_kernel<T>, dim3(n * H), dim3(NT), 0, (hipStream_t)stream, qf, (const T*)q,
+                 hipLaunchKernelGGL(latent_query_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, qf, (const T*)q,
                                     (const T*)q_abs, rope, pos, scale, n, H, dim, rot_dim, rot_n, rank));
     return qsv_launch_status("qsv_latent_query");
 }
