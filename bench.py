@@ -12,6 +12,9 @@ greedy sampling, replayed from a hipGraph.  N > 1 = tensor parallel over N GPUs 
 weights, 2 RCCL all-reduces per layer); default WEAK scaling (64 sequences per GPU, `--scaling strong` keeps the
 global batch).  `python bench.py --gpus N` without a launcher re-executes itself under torch.distributed.run.
 
+`--design vekalorn` runs another workload altogether (prompt-phase and decode throughput of a design served by the paged engine
+beside this Llama engine at equal size, one JSON line per size: qserve_amd/serving/bench.py); the default line is unchanged.
+
 `--config` selects the other BASELINE.json configurations (3: g128 bs=128; 4: Qwen1.5-72B TP=8 global bs=64, strong;
 5: KV8, 8k context, bs=8); they are parity-test cases first and bench lines only on request.
 

@@ -23,16 +23,14 @@ def main(argv=None):
     ap.add_argument("--max-tokens", type=int, required=True)
     ap.add_argument("--max-seqs", type=int, default=4)
     ap.add_argument("--device", default="cuda:0")
-    ap.add_argument("--backend", default="hip", choices=["hip", "unfused"], help=argparse.SUPPRESS)
     a = ap.parse_args(argv)
     import torch
 
     from .engine import Engine
-    if a.backend == "hip" and not torch.cuda.is_available():
+    if not torch.cuda.is_available():
         print("trace_run: no GPU visible (served models have no CPU path)", file=sys.stderr)
         return 4
-    eng = Engine.from_pretrained(a.model, dtype=a.dtype, device=a.device if a.backend == "hip" else "cpu",
-                                 max_tokens=a.max_tokens, max_seqs=a.max_seqs, backend=a.backend)
+    eng = Engine.from_pretrained(a.model, dtype=a.dtype, device=a.device, max_tokens=a.max_tokens, max_seqs=a.max_seqs)
     os.makedirs(a.out, exist_ok=True)
     slots = {}
     for line in sys.stdin:
