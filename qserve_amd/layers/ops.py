@@ -107,7 +107,9 @@ class HipOps:
             # few workgroups and long contexts (decoding): cut the keys over several workgroups, merged by a second launch
             groups = tiles.size(0) * ((H + 31) // 32)
             span = min(batch.max_pos + 1, int(window)) if window else batch.max_pos + 1
-            splits = max(1, min(self.attention_split_target // max(groups, 1), span // 128, 32)) if key_splits is None else key_splits
+            # (rows wider than 320 elements: one workgroup per CU at a time - a launch of one round of workgroups is the aim)
+            target = self.attention_split_target // 2 if R > 320 else self.attention_split_target
+            splits = max(1, min(target // max(groups, 1), span // 128, 32)) if key_splits is None else key_splits
             po = pm = None
             if splits > 1:
                 po = torch.empty((splits, T, H, rank), dtype=torch.float32, device=qf.device)
