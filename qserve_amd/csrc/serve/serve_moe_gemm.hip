@@ -1,7 +1,7 @@
 // serve_moe_gemm.hip -- grouped expert products on the bf16 matrix cores for the prompt phase (many tokens per expert).
 //
 // The (token, expert) slots are sorted by expert; a work tile = up to 128 consecutive sorted slots of ONE expert (tile list made
-// by the host from the run lengths).  A workgroup computes 128 weight rows x 128 slots of out[s, n] = act(W[e][n, :] . x(s)):
+// by the host from the run lengths).  A workgroup computes 256 weight rows x 128 slots of out[s, n] = act(W[e][n, :] . x(s)):
 // both operands are contiguous along the reduction, so with the weight rows as the A operand and the slots' inputs as the B
 // operand (v_mfma_f32_16x16x32_bf16) a lane ends up with 4 consecutive n of one slot - an 8-byte store.  The input row of a
 // slot is fetched through an index (the gather into sorted order is part of the load), relu(.)^2 is the epilogue of the first
@@ -15,7 +15,8 @@ typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
-constexpr int BNW = 128;     // weight rows per workgroup (32 per wave)
+constexpr int BNW = 256;     // weight rows per workgroup (64 per wave)
+constexpr int MT = BNW / 64; // 16-row blocks per wave
 constexpr int BS = 128;      // slots per tile
 constexpr int KS = 64;       // reduction elements per step
 constexpr int LS = KS + 8;   // LDS row stride (elements)
@@ -25,7 +26,7 @@ constexpr int NPA = BNW * CPR / 256, NPB = BS * CPR / 256;   // pieces per threa
 __device__ __forceinline__ unsigned pack_bf2(float a, float b) { return (unsigned)f2bf(a) | ((unsigned)f2bf(b) << 16); }
 
 template <bool RELU_SQ>
-__global__ __launch_bounds__(256) void grouped_gemm_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
+__global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
                                                            const int64_t* __restrict__ x_index, int div,
                                                            const bf16_t* __restrict__ W, const int32_t* __restrict__ tiles, int N,
                                                            int K) {
@@ -52,9 +53,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(bf16_t* __restrict__ 
         const int64_t s = s_first + (bok[i] ? row : 0);
         bp[i] = X + (size_t)(x_index ? x_index[s] / div : s) * (size_t)K + cc * 8;
     }
-    v4f acc[2][BS / 16];
+    v4f acc[MT][BS / 16];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < BS / 16; ++nt) acc[mt][nt] = v4f{0.f, 0.f, 0.f, 0.f};
     const v4u zero = {0u, 0u, 0u, 0u};
@@ -84,27 +85,27 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(bf16_t* __restrict__ 
         }
 #pragma unroll
         for (int kk = 0; kk < KS; kk += 32) {
-            v4u a[2];
+            v4u a[MT];
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt) a[mt] = *(const v4u*)(As + (32 * w + 16 * mt + col) * LS + kk + 8 * g4);
+            for (int mt = 0; mt < MT; ++mt) a[mt] = *(const v4u*)(As + (16 * MT * w + 16 * mt + col) * LS + kk + 8 * g4);
 #pragma unroll
             for (int nt = 0; nt < BS / 16; ++nt) {
                 const v4u b = *(const v4u*)(Bs + (16 * nt + col) * LS + kk + 8 * g4);
 #pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
+                for (int mt = 0; mt < MT; ++mt)
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a[mt]), __builtin_bit_cast(bf8, b),
                                                                           acc[mt][nt], 0, 0, 0);
             }
         }
     }
-    // this lane: slot 16 nt + col, weight rows n0 + 32 w + 16 mt + 4 g4 + (0 .. 3)
+    // this lane: slot 16 nt + col, weight rows n0 + 16 MT w + 16 mt + 4 g4 + (0 .. 3)
 #pragma unroll
     for (int nt = 0; nt < BS / 16; ++nt) {
         const int sl = 16 * nt + col;
         if (sl >= ns) continue;
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-            const int n = n0 + 32 * w + 16 * mt + 4 * g4;
+        for (int mt = 0; mt < MT; ++mt) {
+            const int n = n0 + 16 * MT * w + 16 * mt + 4 * g4;
             if (n >= N) continue;                                   // N % 4 == 0: the four rows are inside together
             v4f v = acc[mt][nt];
             if (RELU_SQ) {
