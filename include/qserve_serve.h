@@ -72,13 +72,20 @@ int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int
 
 /* Grouped top-k router: scores = softmax(router . h[t]) over n_experts; the experts form n_groups equal groups of neighbours,
  * a group's score is its largest score, only experts of the best keep_groups groups are eligible; the top_k eligible experts
- * with the largest scores are chosen.  idx [T, top_k] int32, weight [T, top_k] float = their scores (not renormalised). */
-int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, int n_tokens, int width, int n_experts,
-                  int top_k, int n_groups, int keep_groups, int dtype, void* stream);
+ * with the largest scores are chosen.  idx [T, top_k] int32, weight [T, top_k] float = their scores (not renormalised).
+ * bias (may be NULL, [n_experts], storage type) is added to the logits before anything else; renorm != 0 divides the chosen
+ * weights by their sum (= the softmax over the chosen logits only). */
+int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, const void* bias, int renorm, int n_tokens,
+                  int width, int n_experts, int top_k, int n_groups, int keep_groups, int dtype, void* stream);
 
-/* act[t, k] = relu(up[idx[t, k]] . h[t])^2     up: [E, ff, width] -> act [T, top_k, ff] (storage type). */
+/* Activations of the first expert product: QSV_ACT_RELU_SQ relu(z)^2; QSV_ACT_GLU: the weight rows come in pairs (2f = gate,
+ * 2f + 1 = up), output f = silu(gate) * up, and the output is half as wide as the product. */
+#define QSV_ACT_NONE 0
+#define QSV_ACT_RELU_SQ 1
+#define QSV_ACT_GLU 2
+/* act[t, k] = activation(up[idx[t, k]] . h[t])     up: [E, ff, width] -> act [T, top_k, ff or ff / 2] (storage type). */
 int qsv_moe_up(void* act, const void* h, const void* up, const int32_t* idx, int n_tokens, int top_k, int width, int ff,
-               int dtype, void* stream);
+               int activation, int dtype, void* stream);
 
 /* y[t] = sum_k weight[t, k] * down[idx[t, k]] . act[t, k]     down: [E, width, ff] -> y [T, width] (storage type). */
 int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx, const float* weight, int n_tokens,
@@ -90,10 +97,10 @@ int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx,
  *   a[i]   = relu(a[i])^2                                           (in place)
  *   y[t]   = sum_k weight[t, k] * ys[inv[t * top_k + k]]            (sorted rows back, weighted; float accumulation) */
 /* Expert-major form (bfloat16): out[s, r] = act(W[e][r, :] . X[x_index ? x_index[s] / div : s, :]) for the sorted slots
- * s in [offsets[e], offsets[e + 1]) of every expert e; W [n_experts, rows, K]; act = relu^2 (relu_sq != 0) or none.  Every
- * weight is read once per launch.  K a multiple of 8, at most 4096. */
+ * s in [offsets[e], offsets[e + 1]) of every expert e; W [n_experts, rows, K]; act = one of QSV_ACT_* (QSV_ACT_GLU: out is
+ * rows / 2 wide).  Every weight is read once per launch.  K a multiple of 8, at most 4096. */
 int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
-                    int n_experts, int rows, int K, int relu_sq, void* stream);
+                    int n_experts, int rows, int K, int act, void* stream);
 /* Grouped expert product on the bf16 matrix cores (prompt phase): the same out[s, n] for work tiles (expert, first sorted slot,
  * slots <= qsv_grouped_gemm_tile_slots()) listed in tiles int32 [n_tiles, 3]; K a multiple of qsv_grouped_gemm_k_step(), n_rows
  * a multiple of 4, n_tiles <= 65535. */
@@ -105,6 +112,65 @@ int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, i
 int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream);
 int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n_tokens, int top_k, int width,
                     int dtype, void* stream);
+
+
+/* ---- several residual streams, statistics-free norm, token shift (serve_streams.hip) ---------------------------------------- */
+/* x[t, s] = table[tokens[t]] * scale for every stream s     x: float [T, streams, width] */
+int qsv_embed_streams(float* x, const void* table, const int32_t* tokens, float scale, int n_tokens, int streams, int width,
+                      int dtype, void* stream);
+/* h[t] = n_t + (n_before - n_t) * shift,  n_t = tanh(alpha * sum_s w_in[s] x[t, s]) * norm_w + norm_b  (shift == NULL: h = n).
+ * n_before: the previous row of the batch if run_off[t] > 0, else prev[state_rd[t]] (zeros if state_rd[t] < 0); the token with
+ * state_wr[t] >= 0 (the last of its run) stores n_t into prev[state_wr[t]].  prev: float [2 * slots, width]. */
+int qsv_hc_read(void* h, const float* x, const float* w_in, const void* norm_w, const void* norm_b, float alpha,
+                const void* shift, float* prev, const int32_t* run_off, const int32_t* state_rd, const int32_t* state_wr,
+                int n_tokens, int streams, int width, int dtype, void* stream);
+/* x[t, r] <- sum_s mix[s, r] x[t, s] + w_out[r] * y[t] for all r at once (at most 8 streams). */
+int qsv_hc_write(float* x, const void* y, const float* mix, const float* w_out, int n_tokens, int streams, int width, int dtype,
+                 void* stream);
+/* out[r] = tanh(alpha * sum_s x[rows[r], s]) * norm_w + norm_b  (rows == NULL: row r). */
+int qsv_dyt_sum_rows(void* out, const float* x, const int32_t* rows, const void* norm_w, const void* norm_b, float alpha,
+                     int n_rows, int streams, int width, int dtype, void* stream);
+/* out[t] = (rms_norm(a[t]) * wa + rms_norm(b[t]) * wb) / 2 over `width`. */
+int qsv_rms_pair_mean(void* out, const void* a, const void* wa, const void* b, const void* wb, float eps, int n_tokens,
+                      int width, int dtype, void* stream);
+/* out[r, f] = silu(a[r, 2f]) * a[r, 2f + 1]     a: [n_rows, 2 ff] */
+int qsv_glu(void* out, const void* a, int n_rows, int ff, int dtype, void* stream);
+
+/* ---- matrix-state recurrences and the attention beside them (serve_recurrent.hip) ------------------------------------------- */
+/* out[t, c] (float, [T, heads * dim]) = a_log ? exp(-exp(a_log[c / dim]) * softplus(z[t, c] + bias[c]))
+ *                                             : sigmoid(z[t, c] + bias[c]) ^ (1 / tau) */
+int qsv_decay(float* out, const void* z, int64_t z_stride, const void* bias, const float* a_log, float tau, int n_tokens,
+              int heads, int dim, int dtype, void* stream);
+/* Causal convolution over time per channel, then silu, of the columns [off, off + channels) of proj; w float [channels, taps],
+ * the last tap is the current token's.  Inputs before a run's start come from hist[state_rd[t]] (float [2 * slots, taps - 1,
+ * channels], oldest first; zeros if state_rd[t] < 0); the run's last token (state_wr[t] >= 0) writes the new history.  The
+ * first n_unit groups of unit_dim channels are then divided by sqrt(sum of squares + 1e-6).  out: float [T, channels]. */
+int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, int channels, int taps, const float* w,
+                       float* hist, const int32_t* run_off, const int32_t* state_rd, const int32_t* state_wr, int n_unit,
+                       int unit_dim, int n_tokens, int dtype, void* stream);
+/* Per run (slot, first token, tokens, first position) and head, token by token, with S = state[slot, head] (float [dim, vdim],
+ * zeros if the first position is 0) written back at the end, g = decay[t, head]:
+ *   beta == NULL:  S <- diag(g) S + k v^T                                  o = S^T q * q_scale
+ *   else:          S <- diag(g) S;  u = sigmoid(beta[t, head]) (v - S^T k);  S <- S + k u^T;  o = S^T q * q_scale
+ * q, k: [T, qk_heads, dim] (head h reads h / (heads / qk_heads)), v: [T, heads, vdim], each with its row stride, of type
+ * qkv_dtype; o: float [T, heads, vdim]. */
+int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                       int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
+                       int beta_dtype, float* state, const int32_t* runs, int n_runs, int heads, int qk_heads, int dim,
+                       int vdim, float q_scale, void* stream);
+/* out[t, h] = o[t, h] / rms(o[t, h]) * w * gate_fn(gate[t, h]) over vdim; gate_kind 0: silu, 1: sigmoid. */
+int qsv_head_rms_gate(void* out, const float* o, const void* w, const void* gate, int64_t gate_stride, int gate_kind, float eps,
+                      int n_tokens, int heads, int vdim, int dtype, void* stream);
+/* Rotations in the halves layout (pair p of n rotated dimensions = p and p + n / 2; rope: float [positions, 2, n / 2]):
+ *   qf[t, h]           = [ 0 (vdim) | rot_k(q[t, h]) * scale ]            float [T, heads, vdim + dim]
+ *   pool[g, slot[t]]   = [ rot_v(v[t, g]) | rot_k(k[t, g]) ]              [kv_heads, pool_rows, vdim + dim]
+ * rot_k turns the first rot_n of dim dimensions, rot_v all vdim; q, k, v are column ranges of proj. */
+int qsv_attention_prep(float* qf, void* pool, int64_t pool_rows, const void* proj, int64_t stride, int q_off, int k_off, int v_off,
+                       int heads, int kv_heads, int dim, int vdim, int rot_n, const float* rope_k, const float* rope_v,
+                       float scale, const int64_t* slot, const int32_t* pos, int n_tokens, int dtype, void* stream);
+/* o[t, h, 0:n] turned by sign * pos[t], in place. */
+int qsv_rotate_heads(void* o, const float* rope, const int32_t* pos, float sign, int n_tokens, int heads, int n, int dtype,
+                     void* stream);
 
 #ifdef __cplusplus
 }

@@ -80,7 +80,8 @@ def build(force=False, verbose=True, extra=(), timing=False):
 SERVE_CSRC = os.path.join(CSRC, "serve")
 SERVE_BUILD = os.path.join(HERE, "_build_serve")
 SERVE_LIB = os.path.join(HERE, "libqserve_serve.so")
-SERVE_SOURCES = ["serve_rows.hip", "serve_attention.hip", "serve_attention_mfma.hip", "serve_moe.hip", "serve_moe_gemm.hip"]
+SERVE_SOURCES = ["serve_rows.hip", "serve_attention.hip", "serve_attention_mfma.hip", "serve_moe.hip", "serve_moe_gemm.hip",
+                 "serve_streams.hip", "serve_recurrent.hip"]
 # packed-FP32 instructions off: the kernels' float statistics must not depend on how the compiler pairs them
 SERVE_FLAGS = FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

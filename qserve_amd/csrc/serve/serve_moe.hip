@@ -40,8 +40,9 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 // groups and for experts.
 template <typename T>
 __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx, float* __restrict__ weight,
-                                                       const T* __restrict__ h, const T* __restrict__ router, int D, int E,
-                                                       int top_k, int G, int keep) {
+                                                       const T* __restrict__ h, const T* __restrict__ router,
+                                                       const T* __restrict__ bias, int renorm, int D, int E, int top_k, int G,
+                                                       int keep) {
     __shared__ float s[MAX_EXPERTS];
     __shared__ float gs[MAX_EXPERTS];
     __shared__ unsigned char ok[MAX_EXPERTS];
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
             for (int i = lane; i < D; i += 64) d += ld(r, i) * ld(x, i);
         }
         d = wave_sum(d);
-        if (lane == 0) s[e] = d;
+        if (lane == 0) s[e] = bias ? d + ld(bias, e) : d;
     }
     __syncthreads();
     // (the other three waves only keep the barriers company from here on: the selection is a few hundred steps of one wave)
@@ -110,6 +111,7 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
         }
         __syncthreads();
     }
+    float chosen = 0.f;                                     // (lane 0 of the selecting wave: sum of the chosen scores)
     for (int k = 0; k < top_k; ++k) {                       // the top_k eligible experts
         if (sel) {
             float bv = 0.f;
@@ -124,14 +126,27 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
                 ok[bi] = 0;
                 idx[t * top_k + k] = bi;
                 weight[t * top_k + k] = bv;
+                chosen += bv;
             }
         }
         __syncthreads();
     }
+    // weights over the chosen only: p_i / sum of the chosen p = the softmax over the chosen logits
+    if (renorm && sel && lane == 0)
+        for (int k = 0; k < top_k; ++k) weight[t * top_k + k] /= chosen;
 }
 
-// One workgroup per (token, chosen expert): act = relu(up_e . h)^2.  Dynamic LDS: D floats.
-template <typename T>
+// Activation of the first expert product.  ACT_GLU: the weight rows come in pairs (2f = gate, 2f + 1 = up) and output f is
+// silu(gate) * up, so the output is half as wide as the product.
+constexpr int ACT_NONE = 0, ACT_RELU_SQ = 1, ACT_GLU = 2;
+__device__ __forceinline__ float relu_sq(float d) {
+    const float a = fmaxf(d, 0.f);
+    return a * a;
+}
+__device__ __forceinline__ float glu(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// One workgroup per (token, chosen expert): act = relu(up_e . h)^2 (or the gated unit).  Dynamic LDS: D floats.  ff: weight rows.
+template <typename T, int ACT>
 __global__ __launch_bounds__(NT) void moe_up_kernel(T* __restrict__ act, const T* __restrict__ h, const T* __restrict__ up,
                                                     const int32_t* __restrict__ idx, int top_k, int D, int ff) {
     extern __shared__ float xs[];
@@ -141,15 +156,26 @@ __global__ __launch_bounds__(NT) void moe_up_kernel(T* __restrict__ act, const T
     for (int i = threadIdx.x; i < D; i += NT) xs[i] = ld(h, t * D + i);
     __syncthreads();
     const T* W = up + (size_t)idx[slot] * ff * D;
+    if (ACT == ACT_GLU) {
+        for (int f = w; f < ff / 2; f += NW) {
+            const T* r = W + (size_t)(2 * f) * D;
+            float d = 0.f, e = 0.f;
+            for (int i = lane; i < D; i += 64) {
+                d += ld(r, i) * xs[i];
+                e += ld(r, D + i) * xs[i];
+            }
+            d = wave_sum(d);
+            e = wave_sum(e);
+            if (lane == 0) st(act, slot * (ff / 2) + f, glu(d, e));
+        }
+        return;
+    }
     for (int f = w; f < ff; f += NW) {
         const T* r = W + (size_t)f * D;
         float d = 0.f;
         for (int i = lane; i < D; i += 64) d += ld(r, i) * xs[i];
         d = wave_sum(d);
-        if (lane == 0) {
-            const float a = fmaxf(d, 0.f);
-            st(act, slot * ff + f, a * a);
-        }
+        if (lane == 0) st(act, slot * ff + f, relu_sq(d));
     }
 }
 
@@ -179,7 +205,7 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(T* __restrict__ y, const T
 // (the scalar forms above wait for one row's loads before they issue the next row's: latency-bound at real layer sizes).
 constexpr int ROWS = 4;      // output rows a wave works on at once
 
-template <typename T>
+template <typename T, int ACT>
 __global__ __launch_bounds__(NT) void moe_up_vec_kernel(T* __restrict__ act, const T* __restrict__ h, const T* __restrict__ up,
                                                         const int32_t* __restrict__ idx, int top_k, int D, int ff) {
     extern __shared__ float xs[];
@@ -205,12 +231,18 @@ __global__ __launch_bounds__(NT) void moe_up_vec_kernel(T* __restrict__ act, con
                 }
             }
         }
+        float d[ROWS];
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            const float d = wave_sum(acc[r]);
-            if (lane == 0 && f0 + r < ff) {
-                const float a = fmaxf(d, 0.f);
-                st(act, slot * ff + f0 + r, a * a);
+        for (int r = 0; r < ROWS; ++r) d[r] = wave_sum(acc[r]);
+        if (lane == 0) {
+            if (ACT == ACT_GLU) {                               // (ROWS and ff are even: a pair never straddles two waves)
+#pragma unroll
+                for (int r = 0; r < ROWS; r += 2)
+                    if (f0 + r < ff) st(act, slot * (ff / 2) + (f0 + r) / 2, glu(d[r], d[r + 1]));
+            } else {
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r)
+                    if (f0 + r < ff) st(act, slot * ff + f0 + r, relu_sq(d[r]));
             }
         }
     }
@@ -260,7 +292,7 @@ __global__ __launch_bounds__(NT) void moe_down_vec_kernel(T* __restrict__ y, con
 // expert); a wave keeps its four weight rows in registers (packed bfloat16) and walks the tokens routed to the expert, so every
 // weight is read once per step however many tokens share the expert.  No host synchronisation. ----------------------------------
 typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-template <int KI, bool RELU_SQ>
+template <int KI, int ACT>
 __global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
                                                          const int64_t* __restrict__ x_index, int div, const bf16_t* __restrict__ W,
                                                          const int64_t* __restrict__ offsets, int rows, int K) {
@@ -308,15 +340,18 @@ __global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ ou
                 }
             }
             if (sb + j < s1) {                                              // (wave-uniform)
+                float d[ROWS];
 #pragma unroll
-                for (int r = 0; r < ROWS; ++r) {
-                    float d = wave_sum(acc[r]);
-                    if (lane == 0 && r0 + r < rows) {
-                        if (RELU_SQ) {
-                            d = fmaxf(d, 0.f);
-                            d *= d;
-                        }
-                        out[(size_t)(sb + j) * rows + r0 + r] = f2bf(d);
+                for (int r = 0; r < ROWS; ++r) d[r] = wave_sum(acc[r]);
+                if (lane == 0) {
+                    if (ACT == ACT_GLU) {
+#pragma unroll
+                        for (int r = 0; r < ROWS; r += 2)
+                            if (r0 + r < rows) out[(size_t)(sb + j) * (rows / 2) + (r0 + r) / 2] = f2bf(glu(d[r], d[r + 1]));
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < ROWS; ++r)
+                            if (r0 + r < rows) out[(size_t)(sb + j) * rows + r0 + r] = f2bf(ACT == ACT_RELU_SQ ? relu_sq(d[r]) : d[r]);
                     }
                 }
             }
@@ -364,21 +399,25 @@ extern "C" int qsv_gather_rows(void* out, const void* src, const int64_t* order,
     return qsv_launch_status("qsv_gather_rows");
 }
 // out[s, r] = act(W[e][r, :] . X[x_index ? x_index[s] / div : s, :]) for the sorted slots s in [offsets[e], offsets[e + 1]) of every
-// expert e; W [E, rows, K] bfloat16, act = relu^2 or nothing.  K % 8 == 0, K <= 4096.
+// expert e; W [E, rows, K] bfloat16, act: 0 nothing, 1 relu^2, 2 gated unit (row pairs; out is rows / 2 wide).  K % 8 == 0, K <= 4096.
 extern "C" int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
-                               int n_experts, int rows, int K, int relu_sq, void* stream) {
+                               int n_experts, int rows, int K, int act, void* stream) {
     QSV_REQUIRE(out && X && W && offsets && n_experts > 0 && rows > 0 && div > 0, "qsv_expert_rows: bad arguments");
+    QSV_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQ || (act == ACT_GLU && rows % 2 == 0), "qsv_expert_rows: activation %d", act);
     QSV_REQUIRE(K > 0 && K % 8 == 0 && K <= 4096, "qsv_expert_rows: inner width %d (a multiple of 8, at most 4096)", K);
     QSV_REQUIRE(n_experts <= 65535, "qsv_expert_rows: too many experts");
     const dim3 grid((rows + NW * ROWS - 1) / (NW * ROWS), n_experts), block(NT);
 #define QSV_ER(KI)                                                                                                           \
     do {                                                                                                                     \
-        if (relu_sq)                                                                                                         \
-            hipLaunchKernelGGL((expert_rows_kernel<KI, true>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, \
-                               x_index, div, (const bf16_t*)W, offsets, rows, K);                                            \
+        if (act == ACT_RELU_SQ)                                                                                              \
+            hipLaunchKernelGGL((expert_rows_kernel<KI, ACT_RELU_SQ>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out,         \
+                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K);                          \
+        else if (act == ACT_GLU)                                                                                             \
+            hipLaunchKernelGGL((expert_rows_kernel<KI, ACT_GLU>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out,             \
+                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K);                          \
         else                                                                                                                 \
-            hipLaunchKernelGGL((expert_rows_kernel<KI, false>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, \
-                               x_index, div, (const bf16_t*)W, offsets, rows, K);                                            \
+            hipLaunchKernelGGL((expert_rows_kernel<KI, ACT_NONE>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out,            \
+                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K);                          \
     } while (0)
     if (K <= 512) QSV_ER(1);
     else if (K <= 1024) QSV_ER(2);
@@ -405,8 +444,8 @@ extern "C" int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, cons
     return qsv_launch_status("qsv_moe_combine");
 }
 
-extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, int n, int D, int E, int top_k,
-                             int G, int keep, int dtype, void* stream) {
+extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, const void* bias, int renorm, int n,
+                             int D, int E, int top_k, int G, int keep, int dtype, void* stream) {
     QSV_REQUIRE(idx && weight && h && router && n >= 0 && D > 0, "qsv_moe_route: bad arguments");
     QSV_REQUIRE(E > 0 && E <= MAX_EXPERTS && G > 0 && E % G == 0 && keep > 0 && keep <= G && top_k > 0 &&
                     top_k <= keep * (E / G),
@@ -414,23 +453,29 @@ extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const v
     if (n == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_moe_route",
                  hipLaunchKernelGGL(moe_route_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, idx, weight, (const T*)h,
-                                    (const T*)router, D, E, top_k, G, keep));
+                                    (const T*)router, (const T*)bias, renorm, D, E, top_k, G, keep));
     return qsv_launch_status("qsv_moe_route");
 }
 
 extern "C" int qsv_moe_up(void* act, const void* h, const void* up, const int32_t* idx, int n, int top_k, int D, int ff,
-                          int dtype, void* stream) {
+                          int activation, int dtype, void* stream) {
     QSV_REQUIRE(act && h && up && idx && n >= 0 && top_k > 0 && D > 0 && ff > 0, "qsv_moe_up: bad arguments");
+    QSV_REQUIRE(activation == ACT_RELU_SQ || (activation == ACT_GLU && ff % 2 == 0), "qsv_moe_up: activation %d over %d rows",
+                activation, ff);
     QSV_REQUIRE((size_t)D * 4 <= 64 * 1024, "qsv_moe_up: width %d does not fit the workgroup's LDS", D);
     if (n == 0) return QSV_OK;
-    if (D % 8 == 0)
-        QSV_DISPATCH(dtype, "qsv_moe_up",
-                     hipLaunchKernelGGL(moe_up_vec_kernel<T>, dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,
-                                        (const T*)h, (const T*)up, idx, top_k, D, ff));
-    else
-        QSV_DISPATCH(dtype, "qsv_moe_up",
-                     hipLaunchKernelGGL(moe_up_kernel<T>, dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,
-                                        (const T*)h, (const T*)up, idx, top_k, D, ff));
+#define QSV_UP(KERNEL, ACT)                                                                                                  \
+    QSV_DISPATCH(dtype, "qsv_moe_up",                                                                                        \
+                 hipLaunchKernelGGL((KERNEL<T, ACT>), dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,   \
+                                    (const T*)h, (const T*)up, idx, top_k, D, ff))
+    if (D % 8 == 0) {
+        if (activation == ACT_GLU) QSV_UP(moe_up_vec_kernel, ACT_GLU);
+        else QSV_UP(moe_up_vec_kernel, ACT_RELU_SQ);
+    } else {
+        if (activation == ACT_GLU) QSV_UP(moe_up_kernel, ACT_GLU);
+        else QSV_UP(moe_up_kernel, ACT_RELU_SQ);
+    }
+#undef QSV_UP
     return qsv_launch_status("qsv_moe_up");
 }
 

@@ -1,0 +1,330 @@
+// serve_recurrent.hip -- matrix-state recurrences (gated linear attention, gated delta rule) and what feeds them: decays,
+// the short causal convolution with its history state, unit norms, the per-head output norm with its gate; and the rotations of
+// the attention that runs beside them (queries, keys and values in the halves layout, cache rows written in the same pass).
+// Everything that enters a recurrence is float; the state is float in memory and in registers.
+#include "serve_common.h"
+
+namespace {
+constexpr int NT = 256;
+constexpr int NW = NT / 64;
+
+__device__ __forceinline__ float softplusf(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// ---- decays ---------------------------------------------------------------------------------------------------------------
+// mode 0: sigmoid(z + bias)^(1 / tau) = exp(-softplus(-(z + bias)) / tau);  mode 1: exp(-exp(a_log[head]) softplus(z + bias))
+template <typename T>
+__global__ __launch_bounds__(NT) void decay_kernel(float* __restrict__ out, const T* __restrict__ z, int64_t z_stride,
+                                                   const T* __restrict__ bias, const float* __restrict__ a_log, float inv_tau,
+                                                   int dim, int n) {
+    const size_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < n; c += NT) {
+        const float v = ld(z, t * z_stride + c) + ld(bias, c);
+        out[t * n + c] = a_log ? expf(-expf(a_log[c / dim]) * softplusf(v)) : expf(-softplusf(-v) * inv_tau);
+    }
+}
+
+// ---- causal convolution over time + silu, unit norm of the leading groups -----------------------------------------------------
+// Workgroup = token.  Tap j (last column = the current token) reads the input taps - 1 - j tokens back: a row of this batch
+// inside the run, the sequence's history state before the run's start, zero before the sequence's start.  The last token of a
+// run writes the new history (the last taps - 1 inputs) into the state's other copy.  Dynamic LDS: C floats.
+template <typename T>
+__global__ __launch_bounds__(NT) void conv_silu_unit_kernel(float* __restrict__ out, const T* __restrict__ proj, int64_t stride,
+                                                            int off, int C, int taps, const float* __restrict__ w,
+                                                            float* __restrict__ hist, const int32_t* __restrict__ run_off,
+                                                            const int32_t* __restrict__ state_rd,
+                                                            const int32_t* __restrict__ state_wr, int n_unit, int unit_dim) {
+    extern __shared__ float ys[];
+    const size_t t = blockIdx.x;
+    const int i = run_off[t], rd = state_rd[t], wr = state_wr[t];
+    const int past = taps - 1;
+    for (int c = threadIdx.x; c < C; c += NT) {
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int d = past - j;
+            float xv = 0.f;
+            if (d <= i) xv = ld(proj, (t - d) * stride + off + c);
+            else if (rd >= 0) xv = hist[((size_t)rd * past + (past + i - d)) * C + c];
+            acc += w[(size_t)c * taps + j] * xv;
+        }
+        ys[c] = acc / (1.0f + expf(-acc));
+        if (wr >= 0) {
+            for (int jj = 0; jj < past; ++jj) {
+                const int e = i + 1 - past + jj;            // index within the run of the input that becomes history entry jj
+                float xv = 0.f;
+                if (e >= 0) xv = ld(proj, (t - (i - e)) * stride + off + c);
+                else if (rd >= 0) xv = hist[((size_t)rd * past + (jj + i + 1)) * C + c];
+                hist[((size_t)wr * past + jj) * C + c] = xv;
+            }
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int g = wv; g < n_unit; g += NW) {
+        float s = 0.f;
+        for (int e = lane; e < unit_dim; e += 64) s += ys[g * unit_dim + e] * ys[g * unit_dim + e];
+        const float inv = 1.0f / sqrtf(wave_sum(s) + 1e-6f);
+        for (int e = lane; e < unit_dim; e += 64) out[t * C + g * unit_dim + e] = ys[g * unit_dim + e] * inv;
+    }
+    for (int c = n_unit * unit_dim + threadIdx.x; c < C; c += NT) out[t * C + c] = ys[c];
+}
+
+// ---- the recurrence ---------------------------------------------------------------------------------------------------------
+// Columns of S (value channels) never meet: column j of head h needs k, q and the decay of the token and its own v_j.  A wave
+// owns 64 / LPC columns of one (run, head); a lane owns R rows of one column, LPC lanes share a column and exchange their
+// partial dot products by butterflies.  The wave walks the run's tokens in order with the next token's operands already
+// requested; the state is read once before and written once after (a run that starts its sequence starts from zeros).
+template <typename TQ, typename TB, bool DELTA, int R>
+__global__ __launch_bounds__(64) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
+                                                            const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
+                                                            int64_t v_stride, const float* __restrict__ decay,
+                                                            const TB* __restrict__ beta, int64_t beta_stride,
+                                                            float* __restrict__ state, const int32_t* __restrict__ runs, int H,
+                                                            int QH, int dim, int vdim, int lpc, float q_scale) {
+    const int lane = threadIdx.x;
+    const int cols = 64 / lpc;
+    const int part = lane / cols, j = blockIdx.z * cols + lane % cols;
+    const bool col_ok = j < vdim;
+    const int r0 = part * R;
+    const int slot = runs[4 * blockIdx.x], first = runs[4 * blockIdx.x + 1], n = runs[4 * blockIdx.x + 2];
+    const bool fresh = runs[4 * blockIdx.x + 3] == 0;
+    const int h = blockIdx.y, qh = h / (H / QH);
+    float* Sg = state + (((size_t)slot * H + h) * dim) * (size_t)vdim + (col_ok ? j : 0);
+    float S[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) S[i] = (!fresh && col_ok && r0 + i < dim) ? Sg[(size_t)(r0 + i) * vdim] : 0.f;
+
+    float kc[R], qc[R], gc[R], vc, bc = 0.f;
+    auto load = [&](int t, float (&kk)[R], float (&qq)[R], float (&gg)[R], float& vv, float& bb) {
+        const TQ* kr = k + (size_t)t * k_stride + (size_t)qh * dim;
+        const TQ* qr = q + (size_t)t * q_stride + (size_t)qh * dim;
+        const float* gr = decay + ((size_t)t * H + h) * (size_t)dim;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const bool ok = r0 + i < dim;
+            kk[i] = ok ? ld(kr, r0 + i) : 0.f;
+            qq[i] = ok ? ld(qr, r0 + i) : 0.f;
+            gg[i] = ok ? gr[r0 + i] : 0.f;
+        }
+        vv = col_ok ? ld(v, (size_t)t * v_stride + (size_t)h * vdim + j) : 0.f;
+        if (DELTA) bb = ld(beta, (size_t)t * beta_stride + h);
+    };
+    load(first, kc, qc, gc, vc, bc);
+    for (int t = first; t < first + n; ++t) {
+        float kn[R], qn[R], gn[R], vn = 0.f, bn = 0.f;
+        if (t + 1 < first + n) load(t + 1, kn, qn, gn, vn, bn);        // (wave-uniform)
+        float acc = 0.f;
+        if (DELTA) {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                S[i] *= gc[i];
+                acc += S[i] * kc[i];
+            }
+            for (int m = cols; m < 64; m <<= 1) acc += __shfl_xor(acc, m, 64);
+            const float u = (vc - acc) / (1.0f + expf(-bc));
+            acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                S[i] += kc[i] * u;
+                acc += S[i] * qc[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                S[i] = gc[i] * S[i] + kc[i] * vc;
+                acc += S[i] * qc[i];
+            }
+        }
+        for (int m = cols; m < 64; m <<= 1) acc += __shfl_xor(acc, m, 64);
+        if (part == 0 && col_ok) o[((size_t)t * H + h) * (size_t)vdim + j] = acc * q_scale;
+        if (t + 1 < first + n) {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                kc[i] = kn[i];
+                qc[i] = qn[i];
+                gc[i] = gn[i];
+            }
+            vc = vn;
+            bc = bn;
+        }
+    }
+    if (col_ok) {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+            if (r0 + i < dim) Sg[(size_t)(r0 + i) * vdim] = S[i];
+    }
+}
+
+// ---- per-head RMS norm of the read-out, times a weight shared by the heads, times a gate ---------------------------------------
+// gate_kind 0: silu(g), 1: sigmoid(g)
+template <typename T>
+__global__ __launch_bounds__(NT) void head_rms_gate_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ w,
+                                                           const T* __restrict__ gate, int64_t gate_stride, int gate_kind, float eps,
+                                                           int H, int vdim) {
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int h = wv; h < H; h += NW) {
+        const float* oh = o + (t * H + h) * (size_t)vdim;
+        float s = 0.f;
+        for (int e = lane; e < vdim; e += 64) s += oh[e] * oh[e];
+        const float inv = 1.0f / sqrtf(wave_sum(s) / (float)vdim + eps);
+        for (int e = lane; e < vdim; e += 64) {
+            const float g = ld(gate, t * gate_stride + (size_t)h * vdim + e);
+            const float sg = 1.0f / (1.0f + expf(-g));
+            st(out, (t * H + h) * (size_t)vdim + e, oh[e] * inv * ld(w, e) * (gate_kind == 0 ? g * sg : sg));
+        }
+    }
+}
+
+// ---- rotations, halves layout: pair p of n rotated dimensions = (p, p + n / 2); rope [positions, 2, n / 2] -------------------
+__device__ __forceinline__ float rot_halves(float u_lo, float u_hi, bool upper, float c, float s) {
+    return upper ? u_hi * c + u_lo * s : u_lo * c - u_hi * s;
+}
+template <typename T>
+__device__ __forceinline__ float rotated(const T* vec, int d, int n, const float* cs) {   // element d of the rotated vector
+    if (d >= n) return ld(vec, d);
+    const int half = n >> 1, p = d < half ? d : d - half;
+    return rot_halves(ld(vec, p), ld(vec, p + half), d >= half, cs[p], cs[half + p]);
+}
+
+// qf[t, h] = [0 (vdim) | rot(q[t, h]) * scale]; pool[g, slot[t]] = [rot_v(v[t, g]) | rot(k[t, g])]
+template <typename T>
+__global__ __launch_bounds__(NT) void attention_prep_kernel(float* __restrict__ qf, T* __restrict__ pool, int64_t pool_rows,
+                                                            const T* __restrict__ proj, int64_t stride, int q_off, int k_off,
+                                                            int v_off, int H, int G, int dim, int vdim, int rot_n,
+                                                            const float* __restrict__ rope_k, const float* __restrict__ rope_v,
+                                                            float scale, const int64_t* __restrict__ slot,
+                                                            const int32_t* __restrict__ pos) {
+    const size_t t = blockIdx.x;
+    const int R = vdim + dim, p = pos[t];
+    const T* row = proj + t * stride;
+    const float* ck = rope_k + (size_t)p * rot_n;
+    const float* cv = rope_v + (size_t)p * vdim;
+    for (int idx = threadIdx.x; idx < H * R; idx += NT) {
+        const int h = idx / R, c = idx - h * R;
+        qf[t * H * (size_t)R + idx] = c < vdim ? 0.f : rotated(row + q_off + h * dim, c - vdim, rot_n, ck) * scale;
+    }
+    for (int idx = threadIdx.x; idx < G * R; idx += NT) {
+        const int g = idx / R, c = idx - g * R;
+        const float val = c < vdim ? rotated(row + v_off + g * vdim, c, vdim, cv) : rotated(row + k_off + g * dim, c - vdim, rot_n, ck);
+        st(pool, ((size_t)g * pool_rows + (size_t)slot[t]) * R + c, val);
+    }
+}
+
+// o[t, h, :n] turned by sign * pos[t] in place
+template <typename T>
+__global__ __launch_bounds__(NT) void rotate_heads_kernel(T* __restrict__ o, const float* __restrict__ rope,
+                                                          const int32_t* __restrict__ pos, float sign, int H, int n) {
+    const size_t t = blockIdx.x;
+    const int half = n >> 1;
+    const float* cs = rope + (size_t)pos[t] * n;
+    for (int idx = threadIdx.x; idx < H * half; idx += NT) {
+        const int h = idx / half, p = idx - h * half;
+        T* vec = o + (t * H + h) * (size_t)n;
+        const float a = ld(vec, p), b = ld(vec, p + half), c = cs[p], s = cs[half + p] * sign;
+        st(vec, p, a * c - b * s);
+        st(vec, p + half, b * c + a * s);
+    }
+}
+}  // namespace
+
+extern "C" int qsv_decay(float* out, const void* z, int64_t z_stride, const void* bias, const float* a_log, float tau, int n_tokens,
+                         int heads, int dim, int dtype, void* stream) {
+    QSV_REQUIRE(out && z && bias && n_tokens >= 0 && heads > 0 && dim > 0 && z_stride >= (int64_t)heads * dim,
+                "qsv_decay: bad arguments");
+    QSV_REQUIRE(a_log || tau > 0.f, "qsv_decay: a power-sigmoid decay needs tau > 0");
+    if (n_tokens == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_decay",
+                 hipLaunchKernelGGL(decay_kernel<T>, dim3(n_tokens), dim3(NT), 0, (hipStream_t)stream, out, (const T*)z, z_stride,
+                                    (const T*)bias, a_log, a_log ? 0.f : 1.0f / tau, dim, heads * dim));
+    return qsv_launch_status("qsv_decay");
+}
+
+extern "C" int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, int channels, int taps, const float* w,
+                                  float* hist, const int32_t* run_off, const int32_t* state_rd, const int32_t* state_wr,
+                                  int n_unit, int unit_dim, int n_tokens, int dtype, void* stream) {
+    QSV_REQUIRE(out && proj && w && hist && run_off && state_rd && state_wr, "qsv_conv_silu_unit: null argument");
+    QSV_REQUIRE(channels > 0 && taps >= 1 && off >= 0 && off + channels <= stride && n_unit >= 0 && unit_dim > 0 &&
+                    (int64_t)n_unit * unit_dim <= channels && n_tokens >= 0,
+                "qsv_conv_silu_unit: bad sizes");
+    QSV_REQUIRE((size_t)channels * 4 <= 64 * 1024, "qsv_conv_silu_unit: %d channels do not fit the workgroup's LDS", channels);
+    if (n_tokens == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_conv_silu_unit",
+                 hipLaunchKernelGGL(conv_silu_unit_kernel<T>, dim3(n_tokens), dim3(NT), (size_t)channels * 4, (hipStream_t)stream, out,
+                                    (const T*)proj, stride, off, channels, taps, w, hist, run_off, state_rd, state_wr, n_unit,
+                                    unit_dim));
+    return qsv_launch_status("qsv_conv_silu_unit");
+}
+
+extern "C" int qsv_recurrent_scan_rows(void) { return 16; }
+
+extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                  int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
+                                  int beta_dtype, float* state, const int32_t* runs, int n_runs, int heads, int qk_heads, int dim,
+                                  int vdim, float q_scale, void* stream) {
+    constexpr int R = 16;
+    QSV_REQUIRE(o && q && k && v && decay && state && runs, "qsv_recurrent_scan: null argument");
+    QSV_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dim > 0 && dim <= 64 * R && vdim > 0 && n_runs >= 0 &&
+                    heads <= 65535,
+                "qsv_recurrent_scan: bad sizes (%d heads over %d, state %d x %d)", heads, qk_heads, dim, vdim);
+    if (n_runs == 0) return QSV_OK;
+    int lpc = 1;
+    while (lpc * R < dim) lpc <<= 1;
+    const int cols = 64 / lpc;
+    const dim3 grid(n_runs, heads, (vdim + cols - 1) / cols), block(64);
+    QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
+#define QSV_SCAN(TQ, TB, DELTA)                                                                                              \
+    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, R>), grid, block, 0, (hipStream_t)stream, o, (const TQ*)q, q_stride, \
+                       (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state, runs, heads,  \
+                       qk_heads, dim, vdim, lpc, q_scale)
+    if (beta) {
+        if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_SCAN(float, float, true);
+        else if (qkv_dtype == QSV_F32 && beta_dtype == QSV_BF16) QSV_SCAN(float, bf16_t, true);
+        else if (qkv_dtype == QSV_BF16 && beta_dtype == QSV_BF16) QSV_SCAN(bf16_t, bf16_t, true);
+        else QSV_REQUIRE(false, "qsv_recurrent_scan: operand types %d / %d", qkv_dtype, beta_dtype);
+    } else {
+        if (qkv_dtype == QSV_F32) QSV_SCAN(float, float, false);
+        else if (qkv_dtype == QSV_BF16) QSV_SCAN(bf16_t, bf16_t, false);
+        else QSV_REQUIRE(false, "qsv_recurrent_scan: operand type %d", qkv_dtype);
+    }
+#undef QSV_SCAN
+    return qsv_launch_status("qsv_recurrent_scan");
+}
+
+extern "C" int qsv_head_rms_gate(void* out, const float* o, const void* w, const void* gate, int64_t gate_stride, int gate_kind,
+                                 float eps, int n_tokens, int heads, int vdim, int dtype, void* stream) {
+    QSV_REQUIRE(out && o && w && gate && n_tokens >= 0 && heads > 0 && vdim > 0 && gate_stride >= (int64_t)heads * vdim &&
+                    (gate_kind == 0 || gate_kind == 1),
+                "qsv_head_rms_gate: bad arguments");
+    if (n_tokens == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_head_rms_gate",
+                 hipLaunchKernelGGL(head_rms_gate_kernel<T>, dim3(n_tokens), dim3(NT), 0, (hipStream_t)stream, (T*)out, o, (const T*)w,
+                                    (const T*)gate, gate_stride, gate_kind, eps, heads, vdim));
+    return qsv_launch_status("qsv_head_rms_gate");
+}
+
+extern "C" int qsv_attention_prep(float* qf, void* pool, int64_t pool_rows, const void* proj, int64_t stride, int q_off, int k_off,
+                                  int v_off, int heads, int kv_heads, int dim, int vdim, int rot_n, const float* rope_k,
+                                  const float* rope_v, float scale, const int64_t* slot, const int32_t* pos, int n_tokens,
+                                  int dtype, void* stream) {
+    QSV_REQUIRE(qf && pool && proj && rope_k && rope_v && slot && pos, "qsv_attention_prep: null argument");
+    QSV_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0 && vdim % 2 == 0 && rot_n >= 0 && rot_n % 2 == 0 && rot_n <= dim &&
+                    q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + (int64_t)heads * dim <= stride &&
+                    k_off + (int64_t)kv_heads * dim <= stride && v_off + (int64_t)kv_heads * vdim <= stride && n_tokens >= 0,
+                "qsv_attention_prep: bad sizes");
+    if (n_tokens == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_attention_prep",
+                 hipLaunchKernelGGL(attention_prep_kernel<T>, dim3(n_tokens), dim3(NT), 0, (hipStream_t)stream, qf, (T*)pool, pool_rows,
+                                    (const T*)proj, stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim, rot_n, rope_k, rope_v,
+                                    scale, slot, pos));
+    return qsv_launch_status("qsv_attention_prep");
+}
+
+extern "C" int qsv_rotate_heads(void* o, const float* rope, const int32_t* pos, float sign, int n_tokens, int heads, int n,
+                                int dtype, void* stream) {
+    QSV_REQUIRE(o && rope && pos && n_tokens >= 0 && heads > 0 && n > 0 && n % 2 == 0, "qsv_rotate_heads: bad arguments");
+    if (n_tokens == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_rotate_heads",
+                 hipLaunchKernelGGL(rotate_heads_kernel<T>, dim3(n_tokens), dim3(NT), 0, (hipStream_t)stream, (T*)o, rope, pos, sign,
+                                    heads, n));
+    return qsv_launch_status("qsv_rotate_heads");
+}

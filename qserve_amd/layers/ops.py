@@ -133,29 +133,166 @@ class HipOps:
                    "sigmoid_gate")
         return o
 
-    def moe_route(self, h, router, top_k, groups, keep):
+    # ---- streams, position-free norm, token shift -----------------------------------------------------------------------------
+    def embed_streams(self, tokens, table, scale, streams):
+        T, D = tokens.numel(), table.size(1)
+        x = torch.empty((T, streams, D), dtype=torch.float32, device=table.device)
+        self._need(tokens, table)
+        self.check(self.L.qsv_embed_streams(x.data_ptr(), table.data_ptr(), tokens.data_ptr(), float(scale), T, streams, D, self.code,
+                                            self._s()), "embed_streams")
+        return x
+
+    def hc_read(self, x, w_in, norm, shift=None, batch=None, prev=None):
+        """-> the sublayer's input [T, D] (storage type): norm(sum_s w_in[s] x[:, s]), token-shifted if `shift` is given (then
+        `prev` is the sequences' two-copy state [2 slots, D] and `batch` names each token's run and state rows)."""
+        w, b, alpha = norm
+        T, S, D = x.shape
+        h = torch.empty((T, D), dtype=self.dtype, device=x.device)
+        self._need(x, w_in, w, b, shift, prev)
+        assert x.dtype == torch.float32 and w_in.dtype == torch.float32 and w_in.numel() == S
+        p = [0, 0, 0, 0, 0]
+        if shift is not None:
+            assert prev.dtype == torch.float32 and prev.size(-1) == D and shift.dtype == self.dtype
+            p = [shift.data_ptr(), prev.data_ptr(), batch.run_off.data_ptr(), batch.state_rd.data_ptr(), batch.state_wr.data_ptr()]
+        self.check(self.L.qsv_hc_read(h.data_ptr(), x.data_ptr(), w_in.data_ptr(), w.data_ptr(), b.data_ptr(), float(alpha), *p,
+                                      T, S, D, self.code, self._s()), "hc_read")
+        return h
+
+    def hc_write(self, x, y, w_mix, w_out):
+        T, S, D = x.shape
+        self._need(x, y, w_mix, w_out)
+        assert y.shape == (T, D) and y.dtype == self.dtype and w_mix.dtype == torch.float32 and w_mix.shape == (S, S)
+        self.check(self.L.qsv_hc_write(x.data_ptr(), y.data_ptr(), w_mix.data_ptr(), w_out.data_ptr(), T, S, D, self.code, self._s()),
+                   "hc_write")
+        return x
+
+    def dyt_sum_rows(self, x, rows, norm):
+        w, b, alpha = norm
+        T, S, D = x.shape
+        n = T if rows is None else rows.numel()
+        out = torch.empty((n, D), dtype=self.dtype, device=x.device)
+        self._need(x, rows, w, b)
+        self.check(self.L.qsv_dyt_sum_rows(out.data_ptr(), x.data_ptr(), 0 if rows is None else rows.data_ptr(), w.data_ptr(),
+                                           b.data_ptr(), float(alpha), n, S, D, self.code, self._s()), "dyt_sum_rows")
+        return out
+
+    def rms_pair_mean(self, a, wa, b, wb, eps):
+        out = torch.empty_like(a)
+        self._need(a, wa, b, wb)
+        assert a.shape == b.shape and a.dtype == self.dtype and b.dtype == self.dtype
+        self.check(self.L.qsv_rms_pair_mean(out.data_ptr(), a.data_ptr(), wa.data_ptr(), b.data_ptr(), wb.data_ptr(), eps, a.size(0),
+                                            a.size(1), self.code, self._s()), "rms_pair_mean")
+        return out
+
+    def glu(self, a):
+        """a [n, 2 ff] with (gate, up) as neighbours -> silu(gate) * up [n, ff]."""
+        n, ff = a.size(0), a.size(1) // 2
+        out = torch.empty((n, ff), dtype=self.dtype, device=a.device)
+        self._need(a)
+        self.check(self.L.qsv_glu(out.data_ptr(), a.data_ptr(), n, ff, self.code, self._s()), "glu")
+        return out
+
+    # ---- attention with rotated keys and values: rotations + cache write ---------------------------------------------------------
+    def attention_prep(self, proj, q_off, k_off, v_off, heads, kv_heads, dim, vdim, rot_n, rope_k, rope_v, scale, pool, batch):
+        T = proj.size(0)
+        qf = torch.empty((T, heads, vdim + dim), dtype=torch.float32, device=proj.device)
+        self._need(proj, rope_k, rope_v, pool, batch.slot, batch.pos)
+        assert pool.shape[0] == kv_heads and pool.shape[2] == vdim + dim and pool.dtype == self.dtype and proj.dtype == self.dtype
+        assert rope_k.size(-1) * 2 == rot_n and rope_v.size(-1) * 2 == vdim and rope_k.size(0) > batch.max_pos < rope_v.size(0)
+        self.check(self.L.qsv_attention_prep(qf.data_ptr(), pool.data_ptr(), pool.size(1), proj.data_ptr(), proj.stride(0), q_off,
+                                             k_off, v_off, heads, kv_heads, dim, vdim, rot_n, rope_k.data_ptr(), rope_v.data_ptr(),
+                                             float(scale), batch.slot.data_ptr(), batch.pos.data_ptr(), T, self.code, self._s()),
+                   "attention_prep")
+        return qf
+
+    def rotate_heads(self, o, rope, pos, sign):
+        T, H, n = o.shape
+        self._need(o, rope, pos)
+        assert rope.size(-1) * 2 == n and o.dtype == self.dtype
+        self.check(self.L.qsv_rotate_heads(o.data_ptr(), rope.data_ptr(), pos.data_ptr(), float(sign), T, H, n, self.code, self._s()),
+                   "rotate_heads")
+        return o
+
+    # ---- recurrences ----------------------------------------------------------------------------------------------------------
+    def decay(self, z, bias, a_log, tau, heads, dim):
+        """z [T, heads * dim] (storage type; a column slice is fine) -> float decays: a_log given: exp(-exp(a_log[h]) softplus(z +
+        bias)); else sigmoid(z + bias)^(1 / tau)."""
+        T = z.size(0)
+        out = torch.empty((T, heads * dim), dtype=torch.float32, device=z.device)
+        self._need(bias, a_log)
+        assert z.stride(1) == 1 and z.size(1) == heads * dim and z.dtype == self.dtype and bias.dtype == self.dtype
+        assert a_log is None or (a_log.dtype == torch.float32 and a_log.numel() == heads)
+        self.check(self.L.qsv_decay(out.data_ptr(), z.data_ptr(), z.stride(0), bias.data_ptr(), 0 if a_log is None else a_log.data_ptr(),
+                                    float(tau), T, heads, dim, self.code, self._s()), "decay")
+        return out
+
+    def conv_silu_unit(self, proj, off, conv_w, hist, batch, n_unit, unit_dim):
+        T = proj.size(0)
+        C, taps = conv_w.shape
+        out = torch.empty((T, C), dtype=torch.float32, device=proj.device)
+        self._need(proj, conv_w, hist)
+        assert conv_w.dtype == torch.float32 and hist.dtype == torch.float32 and hist.size(-1) == C and proj.dtype == self.dtype
+        assert hist.size(1) == max(taps - 1, 1)
+        self.check(self.L.qsv_conv_silu_unit(out.data_ptr(), proj.data_ptr(), proj.stride(0), off, C, taps, conv_w.data_ptr(),
+                                             hist.data_ptr(), batch.run_off.data_ptr(), batch.state_rd.data_ptr(),
+                                             batch.state_wr.data_ptr(), n_unit, unit_dim, T, self.code, self._s()), "conv_silu_unit")
+        return out
+
+    def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale):
+        """q, k [T, qk_heads * dim], v [T, heads * vdim] (float or storage type, column slices are fine), decay float [T, heads *
+        dim], beta [T, heads] raw (before the sigmoid) or None, state float [slots, heads, dim, vdim] -> o float [T, heads, vdim]."""
+        T = q.size(0)
+        o = torch.empty((T, heads, vdim), dtype=torch.float32, device=q.device)
+        self._need(decay, state)
+        assert q.dtype == k.dtype == v.dtype and q.stride(1) == k.stride(1) == v.stride(1) == 1
+        assert state.shape[1:] == (heads, dim, vdim) and state.dtype == torch.float32 and decay.shape == (T, heads * dim)
+        runs = batch.runs()
+        self.check(self.L.qsv_recurrent_scan(o.data_ptr(), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(),
+                                             v.stride(0), dtype_code(q.dtype), decay.data_ptr(),
+                                             0 if beta is None else beta.data_ptr(), 0 if beta is None else beta.stride(0),
+                                             0 if beta is None else dtype_code(beta.dtype), state.data_ptr(), runs.data_ptr(),
+                                             runs.size(0), heads, qk_heads, dim, vdim, float(q_scale), self._s()), "recurrent_scan")
+        return o
+
+    def head_rms_gate(self, o, w, gate, kind, eps):
+        T, H, dv = o.shape
+        out = torch.empty((T, H * dv), dtype=self.dtype, device=o.device)
+        self._need(o, w)
+        assert gate.stride(1) == 1 and gate.size(1) == H * dv and gate.dtype == self.dtype and w.dtype == self.dtype
+        self.check(self.L.qsv_head_rms_gate(out.data_ptr(), o.data_ptr(), w.data_ptr(), gate.data_ptr(), gate.stride(0),
+                                            {"silu": 0, "sigmoid": 1}[kind], eps, T, H, dv, self.code, self._s()), "head_rms_gate")
+        return out
+
+    def moe_route(self, h, router, top_k, groups, keep, bias=None, renorm=False):
         T, E = h.size(0), router.size(0)
         idx = torch.empty((T, top_k), dtype=torch.int32, device=h.device)
         wt = torch.empty((T, top_k), dtype=torch.float32, device=h.device)
-        self._need(h, router)
-        self.check(self.L.qsv_moe_route(idx.data_ptr(), wt.data_ptr(), h.data_ptr(), router.data_ptr(), T, h.size(1), E, top_k,
+        self._need(h, router, bias)
+        assert bias is None or (bias.dtype == self.dtype and bias.numel() == E)
+        self.check(self.L.qsv_moe_route(idx.data_ptr(), wt.data_ptr(), h.data_ptr(), router.data_ptr(),
+                                        0 if bias is None else bias.data_ptr(), int(bool(renorm)), T, h.size(1), E, top_k,
                                         groups, keep, self.code, self._s()), "moe_route")
         return idx, wt
 
-    def moe_experts(self, h, up, down, idx, wt):
-        """up [E, ff, D], down [E, D, ff]; y[t] = sum_k wt[t, k] * down[idx[t, k]] relu(up[idx[t, k]] h[t])^2."""
+    ACTS = {"none": 0, "relu_sq": 1, "swiglu": 2}
+
+    def moe_experts(self, h, up, down, idx, wt, act="relu_sq"):
+        """up [E, rows, D], down [E, D, ff]; y[t] = sum_k wt[t, k] * down[idx[t, k]] a(up[idx[t, k]] h[t]).  act "relu_sq":
+        a = relu(.)^2, rows = ff; "swiglu": up's rows come in pairs (2f = gate, 2f + 1 = up), a_f = silu(gate_f) up_f, rows = 2 ff."""
         T, D = h.shape
-        top_k, ff = idx.size(1), up.size(1)
+        top_k, rows = idx.size(1), up.size(1)
+        a = self.ACTS[act]
+        ff = rows // 2 if a == 2 else rows
         if (self.code == BF16 and self.moe_token_slots < T * top_k <= self.moe_expert_major_slots and D % 8 == 0 and ff % 8 == 0
                 and D <= 4096 and ff <= 4096):
-            return self._moe_experts_expert_major(h, up, down, idx, wt)
+            return self._moe_experts_expert_major(h, up, down, idx, wt, a)
         if T * top_k > self.moe_sorted_above:
-            return self._moe_experts_sorted(h, up, down, idx, wt)
+            return self._moe_experts_sorted(h, up, down, idx, wt, a)
         act = torch.empty((T, top_k, ff), dtype=self.dtype, device=h.device)
         y = torch.empty((T, D), dtype=self.dtype, device=h.device)
         self._need(h, up, down, idx, wt)
         assert up.shape[2] == D and down.shape == (up.size(0), D, ff)
-        self.check(self.L.qsv_moe_up(act.data_ptr(), h.data_ptr(), up.data_ptr(), idx.data_ptr(), T, top_k, D, ff, self.code,
+        self.check(self.L.qsv_moe_up(act.data_ptr(), h.data_ptr(), up.data_ptr(), idx.data_ptr(), T, top_k, D, rows, a, self.code,
                                      self._s()), "moe_up")
         self.check(self.L.qsv_moe_down(y.data_ptr(), act.data_ptr(), down.data_ptr(), idx.data_ptr(), wt.data_ptr(), T, top_k, D,
                                        ff, self.code, self._s()), "moe_down")
@@ -174,9 +311,10 @@ class HipOps:
     moe_token_slots = 8
     moe_expert_major_slots = 1024
 
-    def _moe_experts_expert_major(self, h, up, down, idx, wt):
+    def _moe_experts_expert_major(self, h, up, down, idx, wt, a=1):
         T, D = h.shape
-        E, ff, K = up.size(0), up.size(1), idx.size(1)
+        E, rows, K = up.size(0), up.size(1), idx.size(1)
+        ff = rows // 2 if a == 2 else rows
         n = T * K
         expert, order = torch.sort(idx.reshape(-1).long(), stable=True)   # order: sorted slot -> slot (t K + k)
         # first sorted slot of every expert (and the end): a search in the sorted list - no count has to reach the host
@@ -186,7 +324,7 @@ class HipOps:
         act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
         ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
         self.check(self.L.qsv_expert_rows(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), offsets.data_ptr(),
-                                          E, ff, D, 1, self._s()), "expert_rows(up)")
+                                          E, rows, D, a, self._s()), "expert_rows(up)")
         self.check(self.L.qsv_expert_rows(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), offsets.data_ptr(), E, D, ff, 0,
                                           self._s()), "expert_rows(down)")
         y = torch.empty((T, D), dtype=self.dtype, device=h.device)
@@ -194,9 +332,11 @@ class HipOps:
                                           self._s()), "moe_combine")
         return y
 
-    def _moe_experts_sorted(self, h, up, down, idx, wt):
+    def _moe_experts_sorted(self, h, up, down, idx, wt, a=1):
+        """a = 2 (gated units): the first product leaves both halves of every unit ([n, 2 ff]), `glu` folds them."""
         T, D = h.shape
-        E, ff, K = up.size(0), up.size(1), idx.size(1)
+        E, rows, K = up.size(0), up.size(1), idx.size(1)
+        ff = rows // 2 if a == 2 else rows
         n = T * K
         flat = idx.reshape(-1)
         order = torch.argsort(flat, stable=True)                       # sorted slot -> slot (t K + k)
@@ -210,12 +350,15 @@ class HipOps:
             for e, c in enumerate(counts):
                 tiles += [(e, a + o, min(ts, c - o)) for o in range(0, c, ts)]
                 a += c
-            act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
+            act = torch.empty((n, rows), dtype=self.dtype, device=h.device)
             ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
-            for lo in range(0, len(tiles), 65535):
-                tl = torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device)
+            tls = [torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device) for lo in range(0, len(tiles), 65535)]
+            for tl in tls:
                 self.check(self.L.qsv_grouped_gemm(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), tl.data_ptr(),
-                                                   tl.size(0), ff, D, 1, self._s()), "grouped_gemm(up)")
+                                                   tl.size(0), rows, D, 1 if a == 1 else 0, self._s()), "grouped_gemm(up)")
+            if a == 2:
+                act = self.glu(act)
+            for tl in tls:
                 self.check(self.L.qsv_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), tl.data_ptr(),
                                                    tl.size(0), D, ff, 0, self._s()), "grouped_gemm(down)")
             y = torch.empty((T, D), dtype=self.dtype, device=h.device)
@@ -225,19 +368,22 @@ class HipOps:
         xs = torch.empty((n, D), dtype=self.dtype, device=h.device)
         self.check(self.L.qsv_gather_rows(xs.data_ptr(), h.data_ptr(), order.data_ptr(), K, n, D, self.code, self._s()),
                    "gather_rows")
-        act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
+        act = torch.empty((n, rows), dtype=self.dtype, device=h.device)
         ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
-        a = 0
+        at = 0
         for e, c in enumerate(counts):
             if c:
-                torch.matmul(xs[a:a + c], up[e].t(), out=act[a:a + c])
-            a += c
-        self.check(self.L.qsv_relu_sq(act.data_ptr(), act.numel(), self.code, self._s()), "relu_sq")
-        a = 0
+                torch.matmul(xs[at:at + c], up[e].t(), out=act[at:at + c])
+            at += c
+        if a == 2:
+            act = self.glu(act)
+        else:
+            self.check(self.L.qsv_relu_sq(act.data_ptr(), act.numel(), self.code, self._s()), "relu_sq")
+        at = 0
         for e, c in enumerate(counts):
             if c:
-                torch.matmul(act[a:a + c], down[e].t(), out=ys[a:a + c])
-            a += c
+                torch.matmul(act[at:at + c], down[e].t(), out=ys[at:at + c])
+            at += c
         y = torch.empty((T, D), dtype=self.dtype, device=h.device)
         self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
                                           self._s()), "moe_combine")
@@ -320,8 +466,124 @@ class TorchOps:
         o.copy_((o.float() * torch.sigmoid(g.float())).to(self.dtype))
         return o
 
-    def moe_route(self, h, router, top_k, groups, keep):
-        s = torch.softmax(h.float() @ router.float().t(), dim=-1)
+    # ---- streams, position-free norm, token shift -----------------------------------------------------------------------------
+    def embed_streams(self, tokens, table, scale, streams):
+        x = table[tokens.long()].float() * scale
+        return x[:, None, :].repeat(1, streams, 1).contiguous()
+
+    def hc_read(self, x, w_in, norm, shift=None, batch=None, prev=None):
+        w, b, alpha = norm
+        n = torch.tanh(alpha * torch.einsum("s,tsd->td", w_in, x)) * w.float() + b.float()
+        if shift is None:
+            return n.to(self.dtype)
+        before = torch.zeros_like(n)
+        before[1:] = n[:-1]
+        for slot, first, cnt in batch.items:
+            rd, wr = int(batch.state_rd[first]), int(batch.state_wr[first + cnt - 1])
+            before[first] = prev[rd] if rd >= 0 else 0.0
+            prev[wr] = n[first + cnt - 1]
+        return (n + (before - n) * shift.float()).to(self.dtype)
+
+    def hc_write(self, x, y, w_mix, w_out):
+        x.copy_(torch.einsum("sr,tsd->trd", w_mix, x) + w_out[None, :, None] * y.float()[:, None, :])
+        return x
+
+    def dyt_sum_rows(self, x, rows, norm):
+        w, b, alpha = norm
+        u = (x if rows is None else x[rows.long()]).sum(1)
+        return (torch.tanh(alpha * u) * w.float() + b.float()).to(self.dtype)
+
+    # ---- rotations in the halves layout (pair i = dimensions i, i + n / 2) ------------------------------------------------------
+    @staticmethod
+    def _rotate_halves(v, rope, pos, n, sign=1.0):
+        cs = rope[pos.long()]
+        c, s = cs[:, 0, None, :], cs[:, 1, None, :] * sign
+        a, b = v[..., :n // 2], v[..., n // 2:n]
+        return torch.cat([a * c - b * s, b * c + a * s, v[..., n:]], dim=-1)
+
+    def attention_prep(self, proj, q_off, k_off, v_off, heads, kv_heads, dim, vdim, rot_n, rope_k, rope_v, scale, pool, batch):
+        T = proj.size(0)
+        q = proj[:, q_off:q_off + heads * dim].float().view(T, heads, dim)
+        k = proj[:, k_off:k_off + kv_heads * dim].float().view(T, kv_heads, dim)
+        v = proj[:, v_off:v_off + kv_heads * vdim].float().view(T, kv_heads, vdim)
+        q = self._rotate_halves(q, rope_k, batch.pos, rot_n) * scale
+        k = self._rotate_halves(k, rope_k, batch.pos, rot_n)
+        v = self._rotate_halves(v, rope_v, batch.pos, vdim)
+        pool[:, batch.slot] = torch.cat([v, k], dim=-1).transpose(0, 1).to(self.dtype)
+        return torch.cat([torch.zeros(T, heads, vdim, device=proj.device), q], dim=-1).contiguous()
+
+    def rotate_heads(self, o, rope, pos, sign):
+        o.copy_(self._rotate_halves(o.float(), rope, pos, o.size(-1), sign).to(self.dtype))
+        return o
+
+    # ---- recurrences ----------------------------------------------------------------------------------------------------------
+    def decay(self, z, bias, a_log, tau, heads, dim):
+        z = z.float() + bias.float()
+        if a_log is None:
+            return torch.exp(-torch.nn.functional.softplus(-z) / tau).contiguous()          # sigmoid(z) ^ (1 / tau)
+        rate = torch.exp(a_log.float()).repeat_interleave(dim)
+        return torch.exp(-rate * torch.nn.functional.softplus(z)).contiguous()
+
+    def conv_silu_unit(self, proj, off, conv_w, hist, batch, n_unit, unit_dim):
+        C, taps = conv_w.shape
+        xin = proj[:, off:off + C].to(self.dtype).float()
+        out = torch.empty_like(xin)
+        w = conv_w.float()
+        for slot, first, cnt in batch.items:
+            rd, wr = int(batch.state_rd[first]), int(batch.state_wr[first + cnt - 1])
+            past = hist[rd] if rd >= 0 else torch.zeros((taps - 1, C), device=xin.device)
+            seq = torch.cat([past, xin[first:first + cnt]])
+            y = sum(seq[j:j + cnt] * w[:, j] for j in range(taps))
+            out[first:first + cnt] = y * torch.sigmoid(y)
+            hist[wr] = seq[cnt:]
+        u = out[:, :n_unit * unit_dim].view(-1, n_unit, unit_dim)
+        out[:, :n_unit * unit_dim] = (u / torch.sqrt((u * u).sum(-1, keepdim=True) + 1e-6)).view(-1, n_unit * unit_dim)
+        return out
+
+    def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale):
+        T = q.size(0)
+        rep = heads // qk_heads
+        qf = q.float().view(T, qk_heads, dim).repeat_interleave(rep, 1) * q_scale
+        kf = k.float().view(T, qk_heads, dim).repeat_interleave(rep, 1)
+        vf, g = v.float().view(T, heads, vdim), decay.view(T, heads, dim)
+        bt = None if beta is None else torch.sigmoid(beta.float())
+        o = torch.empty((T, heads, vdim), dtype=torch.float32, device=q.device)
+        for slot, first, cnt in batch.items:
+            S = state[slot].clone() if int(batch.pos[first]) else torch.zeros_like(state[slot])
+            for t in range(first, first + cnt):
+                S = g[t][:, :, None] * S
+                if bt is None:
+                    S = S + kf[t][:, :, None] * vf[t][:, None, :]
+                else:
+                    u = bt[t][:, None] * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
+                    S = S + kf[t][:, :, None] * u[:, None, :]
+                o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+            state[slot] = S
+        return o
+
+    def head_rms_gate(self, o, w, gate, kind, eps):
+        T, H, dv = o.shape
+        n = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * w.float()
+        g = gate.float().view(T, H, dv)
+        g = g * torch.sigmoid(g) if kind == "silu" else torch.sigmoid(g)
+        return (n * g).reshape(T, H * dv).to(self.dtype)
+
+    def rms_pair_mean(self, a, wa, b, wb, eps):
+        return (0.5 * (self._rms(a, wa, eps) + self._rms(b, wb, eps))).to(self.dtype)
+
+    def glu(self, a):
+        a = a.float()
+        g, u = a[..., 0::2], a[..., 1::2]
+        return (g * torch.sigmoid(g) * u).to(self.dtype)
+
+    def moe_route(self, h, router, top_k, groups, keep, bias=None, renorm=False):
+        z = h.float() @ router.float().t()
+        if bias is not None:
+            z = z + bias.float()
+        if renorm:                                          # weights = softmax over the chosen logits only
+            top = z.topk(top_k, dim=-1)
+            return top.indices.int(), torch.softmax(top.values, dim=-1)
+        s = torch.softmax(z, dim=-1)
         T, E = s.shape
         gs = s.view(T, groups, E // groups).amax(-1)
         kept = torch.zeros_like(gs, dtype=torch.bool).scatter_(1, gs.topk(keep, dim=-1).indices, True)
@@ -329,12 +591,13 @@ class TorchOps:
         idx = s.masked_fill(~ok, -1.0).topk(top_k, dim=-1).indices
         return idx.int(), s.gather(1, idx)
 
-    def moe_experts(self, h, up, down, idx, wt):
+    def moe_experts(self, h, up, down, idx, wt, act="relu_sq"):
         T, D = h.shape
         y = torch.zeros((T, D), dtype=torch.float32, device=h.device)
         for k in range(idx.size(1)):
             e = idx[:, k].long()
-            a = torch.relu(torch.einsum("tfd,td->tf", up[e].float(), h.float())) ** 2
+            a = torch.einsum("tfd,td->tf", up[e].float(), h.float())
+            a = torch.relu(a) ** 2 if act == "relu_sq" else self.glu(a.to(self.dtype)).float()
             a = a.to(self.dtype).float()
             y += wt[:, k, None] * torch.einsum("tdf,tf->td", down[e].float(), a)
         return y.to(self.dtype)

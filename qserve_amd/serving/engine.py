@@ -30,7 +30,19 @@ class StepBatch:
     max_pos: int                # host: largest position in the batch
     n_tokens: int
     items: list = None          # host: [(sequence slot, first flat token index, tokens)] - runs of consecutive positions
+    run_off: torch.Tensor = None    # int32 [T]  index of the token within its run
+    state_rd: torch.Tensor = None   # int32 [T]  two-copy state row the token's run reads (-1: the run starts its sequence)
+    state_wr: torch.Tensor = None   # int32 [T]  two-copy state row to write, on the LAST token of a run (-1 elsewhere)
     _tiles: dict = field(default_factory=dict)
+    _runs: torch.Tensor = None
+
+    def runs(self):
+        """int32 [n_runs, 4] = (sequence slot, first flat token index, tokens, position of the first token), on the device."""
+        if self._runs is None:
+            pos = self.pos.tolist() if self.pos is not None else None
+            rows = [(slot, first, n, pos[first]) for slot, first, n in self.items]
+            self._runs = torch.tensor(rows, dtype=torch.int32).reshape(-1, 4).to(self.pos.device)
+        return self._runs
 
     def tiles(self, tokens_per_tile):
         """Work tiles for kernels that serve a few consecutive tokens of one sequence per workgroup: int32 [n, 3] =
@@ -57,7 +69,7 @@ class Engine:
         self.ops = make_ops(backend, self.dtype, self.device)
         self.model = model_cls.from_config(config, weights, self.ops, self.device, self.dtype, page=page)
         self.cache = PagedCache(self.model.cache_rows, (int(max_tokens) + page - 1) // page, max_seqs, self.dtype, self.device,
-                                page=page)
+                                page=page, states=getattr(self.model, "state_specs", ()))
         self.scheduler = Scheduler(self.cache, max_batch_tokens, prefill_chunk)
         self.requests = {}
         self._ids = itertools.count()
@@ -85,56 +97,70 @@ class Engine:
     def execute(self, items, want):
         """items: [(slot, tokens)] - the next tokens of live sequences, all run as one batch; want: flat indices into the
         concatenated tokens.  -> float logits [len(want), vocab] (None if want is empty)."""
-        toks, seq, pos, rows, runs = [], [], [], [], []
+        toks, seq, pos, rows, runs, off, rd, wr = [], [], [], [], [], [], [], []
         V = self.model.vocab
+        if len({slot for slot, t in items if len(t)}) != sum(1 for _, t in items if len(t)):
+            raise ValueError("a sequence appears twice in one step")
         for slot, t in items:
-            start = self.cache.length[slot]
-            if len(t):
-                runs.append((slot, len(toks), len(t)))
+            start, n = self.cache.length[slot], len(t)
             if any(not 0 <= int(v) < V for v in t):
                 raise ValueError(f"token id outside the vocabulary of {V}")
-            rows += self.cache.extend(slot, len(t))
+            if not n:
+                continue
+            runs.append((slot, len(toks), n))
+            rows += self.cache.extend(slot, n)
             toks += [int(v) for v in t]
-            seq += [slot] * len(t)
-            pos += range(start, start + len(t))
+            seq += [slot] * n
+            pos += range(start, start + n)
+            r, w = self.cache.step_rows(slot)
+            off += range(n)
+            rd += [r if start else -1] * n
+            wr += [-1] * (n - 1) + [w]
         if not toks:
             return None
+        meta = torch.tensor([toks, seq, pos, off, rd, wr], dtype=torch.int32)
         if self.decode_graphs and all(n == 1 for _, _, n in runs):
-            out = self._execute_graph(toks, seq, pos, rows, runs)
+            out = self._execute_graph(meta, rows, runs)
             if out is not None:
                 return out[torch.tensor(list(want), dtype=torch.int64, device=self.device)] if want else None
         dev = self.device
-        # (one host tensor, one copy: int64 rows and int32 metadata share a buffer)
-        meta = torch.tensor([toks, seq, pos], dtype=torch.int32).to(dev)
+        meta = meta.to(dev)
         batch = StepBatch(tokens=meta[0], seq=meta[1], pos=meta[2], slot=torch.tensor(rows, dtype=torch.int64).to(dev),
-                          block_table=self.cache.block_table(), max_pos=max(pos), n_tokens=len(toks), items=runs)
-        x = self.model.forward(batch, self.cache.pools)
+                          block_table=self.cache.block_table(), max_pos=max(pos), n_tokens=len(toks), items=runs,
+                          run_off=meta[3], state_rd=meta[4], state_wr=meta[5])
+        x = self._forward(batch)
         if not want:
             return None
         return self.model.logits(x, torch.tensor(list(want), dtype=torch.int32).to(dev))
 
+    def _forward(self, batch):
+        if self.cache.states:
+            return self.model.forward(batch, self.cache.pools, states=self.cache.states)
+        return self.model.forward(batch, self.cache.pools)
+
     # ---- decode steps from a hipGraph ------------------------------------------------------------------------------------------
     GRAPH_BUCKET = 128                         # positions per context bucket (a graph freezes what is derived from max_pos)
 
-    def _execute_graph(self, toks, seq, pos, rows, runs):
+    def _execute_graph(self, meta, rows, runs):
         """One token per sequence: fill the static inputs of the graph captured for (batch size, context bucket, model
         signature) and replay it.  -> float logits for every row, or None if this shape runs eagerly."""
-        B, dev = len(toks), self.device
-        bucket = max(pos) // self.GRAPH_BUCKET
+        B, dev = meta.size(1), self.device
+        bucket = int(meta[2].max()) // self.GRAPH_BUCKET
         sig = self.model.graph_signature() if hasattr(self.model, "graph_signature") else ()
         key = (B, bucket, sig)
         G = self._graphs.get(key)
         if G is False:
             return None
-        meta = torch.tensor([toks, seq, pos], dtype=torch.int32)
         slot = torch.tensor(rows, dtype=torch.int64)
+        runs4 = torch.tensor([(s, first, n, int(meta[2, first])) for s, first, n in runs], dtype=torch.int32).reshape(-1, 4)
         if G is None:
             if len(self._graphs) >= 16:
                 self._graphs.clear()
             batch = StepBatch(tokens=None, seq=None, pos=None, slot=slot.to(dev), block_table=self.cache.block_table(),
                               max_pos=(bucket + 1) * self.GRAPH_BUCKET - 1, n_tokens=B, items=list(runs))
             m = meta.to(dev)
-            batch.tokens, batch.seq, batch.pos = m[0], m[1], m[2]
+            batch.tokens, batch.seq, batch.pos, batch.run_off, batch.state_rd, batch.state_wr = m[0], m[1], m[2], m[3], m[4], m[5]
+            batch._runs = runs4.to(dev)
             G = {"meta": m, "batch": batch, "rows": torch.arange(B, dtype=torch.int32, device=dev)}
             if hasattr(self.model, "reserve_positions"):
                 self.model.reserve_positions(batch.max_pos + 1)
@@ -142,13 +168,16 @@ class Engine:
             try:
                 side = torch.cuda.Stream()
                 side.wait_stream(torch.cuda.current_stream())
+                kept = [s.clone() for s in self.cache.states]      # a recurrent state must not advance twice: the warm-up's
                 with torch.cuda.stream(side):                      # warm-up outside capture (allocator, lazy initialisation)
-                    self.model.logits(self.model.forward(batch, self.cache.pools), G["rows"])
+                    self.model.logits(self._forward(batch), G["rows"])
                 torch.cuda.current_stream().wait_stream(side)
+                for s, k in zip(self.cache.states, kept):          # ... step is taken back before the replay takes it
+                    s.copy_(k)
                 torch.cuda.synchronize()
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
-                    G["logits"] = self.model.logits(self.model.forward(batch, self.cache.pools), G["rows"])
+                    G["logits"] = self.model.logits(self._forward(batch), G["rows"])
                 G["graph"] = g
             except Exception:                                      # e.g. a launch sequence that synchronises: run eagerly
                 torch.cuda.synchronize()
@@ -158,6 +187,7 @@ class Engine:
         batch = G["batch"]
         G["meta"].copy_(meta)
         batch.slot.copy_(slot)
+        batch._runs.copy_(runs4)
         for tpb, t in batch._tiles.items():
             t.copy_(torch.tensor([(s, first, 1) for s, first, _ in runs], dtype=torch.int32).reshape(-1, 3))
         self.cache.block_table()

@@ -4,8 +4,9 @@ A served model class provides
     from_config(config: dict, weights: dict[name -> tensor], ops, device) -> model
 and the model
     vocab, width          sizes
-    cache_rows            list of cache row widths (elements per token), one per layer that keeps a cache
-    forward(batch, pools) -> float residual stream [T, width] after the last layer
+    cache_rows            list of cache row widths (elements per token; (n, w): n pools of one allocation), one per paged pool
+    state_specs           (optional) list of qserve_amd.serving.cache.StateSpec: fixed-size state per sequence
+    forward(batch, pools[, states=]) -> the float residual stream after the last layer (whatever `logits` reads)
     logits(x, rows)       -> float [len(rows), vocab]
 Families that run through another engine of this package register with `engine=` naming it (see qserve_amd.models).
 """
@@ -14,7 +15,7 @@ import json
 import os
 
 _MODELS = {}
-_BUILTIN = ("qserve_amd.models.vekalorn", "qserve_amd.models.llama_w4a8")
+_BUILTIN = ("qserve_amd.models.vekalorn", "qserve_amd.models.mumelix", "qserve_amd.models.llama_w4a8")
 
 
 def register_model(architecture, engine="paged"):
