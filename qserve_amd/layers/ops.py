@@ -531,11 +531,12 @@ class TorchOps:
         w = conv_w.float()
         for slot, first, cnt in batch.items:
             rd, wr = int(batch.state_rd[first]), int(batch.state_wr[first + cnt - 1])
-            past = hist[rd] if rd >= 0 else torch.zeros((taps - 1, C), device=xin.device)
+            past = hist[rd][:taps - 1] if rd >= 0 else torch.zeros((taps - 1, C), device=xin.device)
             seq = torch.cat([past, xin[first:first + cnt]])
             y = sum(seq[j:j + cnt] * w[:, j] for j in range(taps))
             out[first:first + cnt] = y * torch.sigmoid(y)
-            hist[wr] = seq[cnt:]
+            if taps > 1:
+                hist[wr] = seq[cnt:]
         u = out[:, :n_unit * unit_dim].view(-1, n_unit, unit_dim)
         out[:, :n_unit * unit_dim] = (u / torch.sqrt((u * u).sum(-1, keepdim=True) + 1e-6)).view(-1, n_unit * unit_dim)
         return out

@@ -93,10 +93,9 @@ class Engine:
     def close_sequence(self, slot):
         self.cache.release(slot)
 
-    @torch.no_grad()
-    def execute(self, items, want):
-        """items: [(slot, tokens)] - the next tokens of live sequences, all run as one batch; want: flat indices into the
-        concatenated tokens.  -> float logits [len(want), vocab] (None if want is empty)."""
+    def _layout_host(self, items):
+        """Host side of a step's batch: extends the sequences' pages, swaps their two-copy states.  -> (meta int32 [6, T] =
+        token, slot, position, index in run, state row to read, state row to write; flat cache rows; runs) or None."""
         toks, seq, pos, rows, runs, off, rd, wr = [], [], [], [], [], [], [], []
         V = self.model.vocab
         if len({slot for slot, t in items if len(t)}) != sum(1 for _, t in items if len(t)):
@@ -118,20 +117,38 @@ class Engine:
             wr += [-1] * (n - 1) + [w]
         if not toks:
             return None
-        meta = torch.tensor([toks, seq, pos, off, rd, wr], dtype=torch.int32)
-        if self.decode_graphs and all(n == 1 for _, _, n in runs):
-            out = self._execute_graph(meta, rows, runs)
+        return torch.tensor([toks, seq, pos, off, rd, wr], dtype=torch.int32), rows, runs
+
+    def layout(self, items):
+        """items: [(slot, tokens)] -> the StepBatch of these tokens on the device (None if there are none).  Part of `execute`;
+        callers that run single layers use it directly."""
+        host = self._layout_host(items)
+        return None if host is None else self._to_device(*host)
+
+    def _to_device(self, meta, rows, runs):
+        dev = self.device
+        max_pos = int(meta[2].max())
+        meta = meta.to(dev)                    # (one host tensor, one copy)
+        return StepBatch(tokens=meta[0], seq=meta[1], pos=meta[2], slot=torch.tensor(rows, dtype=torch.int64).to(dev),
+                         block_table=self.cache.block_table(), max_pos=max_pos, n_tokens=meta.size(1), items=runs,
+                         run_off=meta[3], state_rd=meta[4], state_wr=meta[5])
+
+    @torch.no_grad()
+    def execute(self, items, want):
+        """items: [(slot, tokens)] - the next tokens of live sequences, all run as one batch; want: flat indices into the
+        concatenated tokens.  -> float logits [len(want), vocab] (None if want is empty)."""
+        host = self._layout_host(items)
+        if host is None:
+            return None
+        if self.decode_graphs and all(n == 1 for _, _, n in host[2]):
+            out = self._execute_graph(*host)
             if out is not None:
                 return out[torch.tensor(list(want), dtype=torch.int64, device=self.device)] if want else None
-        dev = self.device
-        meta = meta.to(dev)
-        batch = StepBatch(tokens=meta[0], seq=meta[1], pos=meta[2], slot=torch.tensor(rows, dtype=torch.int64).to(dev),
-                          block_table=self.cache.block_table(), max_pos=max(pos), n_tokens=len(toks), items=runs,
-                          run_off=meta[3], state_rd=meta[4], state_wr=meta[5])
+        batch = self._to_device(*host)
         x = self._forward(batch)
         if not want:
             return None
-        return self.model.logits(x, torch.tensor(list(want), dtype=torch.int32).to(dev))
+        return self.model.logits(x, torch.tensor(list(want), dtype=torch.int32).to(self.device))
 
     def _forward(self, batch):
         if self.cache.states:
