@@ -61,11 +61,12 @@ int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
  * index, tokens).  qsv_latent_attention_mfma_ok() says whether the sizes are taken (bfloat16 storage, rank and row width
  * multiples of 8, row width <= 576); otherwise use qsv_latent_attention. * key_splits > 1 cuts every tile's keys over that many workgroups and merges the partial results in a second launch (steps
  * with few tiles: decoding); part_o (float [key_splits, n_tokens, heads, rank]) and part_ml (float [key_splits, n_tokens,
- * heads, 2]) are its workspace. */
+ * heads, 2]) are its workspace.  q_first: every query is zero before this element (0 if unknown); the score product skips the
+ * steps that lie wholly before it. */
 int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                               const int32_t* pos, const int32_t* tiles, int n_tiles, int window, int heads, int rank,
                               int row_width, int page, int key_splits, float* part_o, float* part_ml, int n_tokens,
-                              void* stream);
+                              int q_first, void* stream);
 
 /* o[t, i] *= sigmoid(g[t * g_stride + i]),  i < n. */
 int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int n, int dtype, void* stream);
@@ -124,9 +125,10 @@ int qsv_embed_streams(float* x, const void* table, const int32_t* tokens, float 
 int qsv_hc_read(void* h, const float* x, const float* w_in, const void* norm_w, const void* norm_b, float alpha,
                 const void* shift, float* prev, const int32_t* run_off, const int32_t* state_rd, const int32_t* state_wr,
                 int n_tokens, int streams, int width, int dtype, void* stream);
-/* x[t, r] <- sum_s mix[s, r] x[t, s] + w_out[r] * y[t] for all r at once (at most 8 streams). */
-int qsv_hc_write(float* x, const void* y, const float* mix, const float* w_out, int n_tokens, int streams, int width, int dtype,
-                 void* stream);
+/* x[t, r] <- sum_s mix[s, r] x[t, s] + w_out[r] * y[t] for all r at once (at most 16 streams).  h_next != NULL: also the next
+ * sublayer's input from the new streams, h_next[t] = tanh(alpha * sum_r w_in_next[r] x[t, r]) * norm_w + norm_b (no token shift). */
+int qsv_hc_write(float* x, const void* y, const float* mix, const float* w_out, int n_tokens, int streams, int width, void* h_next,
+                 const float* w_in_next, const void* norm_w, const void* norm_b, float alpha, int dtype, void* stream);
 /* out[r] = tanh(alpha * sum_s x[rows[r], s]) * norm_w + norm_b  (rows == NULL: row r). */
 int qsv_dyt_sum_rows(void* out, const float* x, const int32_t* rows, const void* norm_w, const void* norm_b, float alpha,
                      int n_rows, int streams, int width, int dtype, void* stream);

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     bf16_t* __restrict__ out, const float* __restrict__ qf, const bf16_t* __restrict__ pool,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ pos, const int32_t* __restrict__ tiles,
     int window, int H, int rank, int R, int page, int HP, int TQ, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int n_tokens) {
+    int n_tokens, int s_lo, int s_hi) {
     constexpr int RS = 32 * RT + 8;                      // row stride (elements) of the row-major tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* Ks = (bf16_t*)smem;                          // [BN][RS]
@@ -130,6 +130,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
         v4f sacc[2] = {v4f{0.f, 0.f, 0.f, 0.f}, v4f{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int s = 0; s < RT; ++s) {
+            if (s < s_lo || s >= s_hi) continue;         // (uniform) steps where every query is zero: a leading zero part, padding
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
                 const v4u a = *(const v4u*)(Ks + (16 * mt + col) * RS + 32 * s + 8 * g4);
@@ -300,7 +301,7 @@ extern "C" int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype) 
 extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table,
                                          int table_stride, const int32_t* pos, const int32_t* tiles, int n_tiles, int window,
                                          int H, int rank, int R, int page, int key_splits, float* part_o, float* part_ml,
-                                         int n_tokens, void* stream) {
+                                         int n_tokens, int q_first, void* stream) {
     QSV_REQUIRE(out && qf && pool && block_table && pos && tiles, "qsv_latent_attention_mfma: null argument");
     QSV_REQUIRE(qsv_latent_attention_mfma_ok(rank, R, QSV_BF16) && R >= rank && H > 0 && page > 0 && page % BN == 0 && window >= 0 && n_tiles >= 0,
                 "qsv_latent_attention_mfma: sizes not supported (rank %d, row %d)", rank, R);
@@ -309,7 +310,9 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
     QSV_REQUIRE(key_splits >= 1 && key_splits <= 64 && (key_splits == 1 || (part_o && part_ml && n_tokens > 0)),
                 "qsv_latent_attention_mfma: key splits without workspace");
     const dim3 grid(n_tiles, (H + 15) / 16, key_splits), block(64 * NWV);
+    QSV_REQUIRE(q_first >= 0 && q_first < R, "qsv_latent_attention_mfma: first query element %d of %d", q_first, R);
     const int rt = (R + 31) / 32, ct = (rank + 15) / 16;
+    const int s_lo = q_first / 32, s_hi = rt;
 #define QSV_MFMA(RT, CT)                                                                                                     \
     do {                                                                                                                     \
         size_t lds = (size_t)(BN * (32 * RT + 8) + 16 * CT * VS) * 2;                                                        \
@@ -322,10 +325,11 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
         }                                                                                                                    \
         hipLaunchKernelGGL((latent_attention_mfma_kernel<RT, CT>), grid, block, lds, (hipStream_t)stream, (bf16_t*)out, qf,  \
                            (const bf16_t*)pool, block_table, table_stride, pos, tiles, window, H, rank, R, page, g.HP, g.TQ, \
-                           part_o, part_ml, n_tokens);                                                                       \
+                           part_o, part_ml, n_tokens, s_lo, s_hi);                                                           \
     } while (0)
     if (rt <= 4 && ct <= 8) QSV_MFMA(4, 8);
     else if (rt <= 6 && ct <= 12) QSV_MFMA(6, 12);
+    else if (rt <= 8 && ct <= 8) QSV_MFMA(8, 8);
     else if (rt <= 10 && ct <= 16) QSV_MFMA(10, 16);
     else QSV_MFMA(18, 32);
 #undef QSV_MFMA

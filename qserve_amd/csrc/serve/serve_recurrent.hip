@@ -69,20 +69,50 @@ __global__ __launch_bounds__(NT) void conv_silu_unit_kernel(float* __restrict__ 
 }
 
 // ---- the recurrence ---------------------------------------------------------------------------------------------------------
-// Columns of S (value channels) never meet: column j of head h needs k, q and the decay of the token and its own v_j.  A wave
-// owns 64 / LPC columns of one (run, head); a lane owns R rows of one column, LPC lanes share a column and exchange their
-// partial dot products by butterflies.  The wave walks the run's tokens in order with the next token's operands already
-// requested; the state is read once before and written once after (a run that starts its sequence starts from zeros).
-template <typename TQ, typename TB, bool DELTA, int R>
-__global__ __launch_bounds__(64) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
-                                                            const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
-                                                            int64_t v_stride, const float* __restrict__ decay,
-                                                            const TB* __restrict__ beta, int64_t beta_stride,
-                                                            float* __restrict__ state, const int32_t* __restrict__ runs, int H,
-                                                            int QH, int dim, int vdim, int lpc, float q_scale) {
-    const int lane = threadIdx.x;
-    const int cols = 64 / lpc;
-    const int part = lane / cols, j = blockIdx.z * cols + lane % cols;
+// Columns of S (value channels) never meet: column j of head h needs k, q and the decay of the token and its own v_j.  A
+// workgroup owns a block of columns of one (run, head): a wave 64 / LPC of them, a lane R rows of one column; the LPC lanes of a
+// column are neighbours and add their partial dot products through DPP moves.  The run's tokens are walked in order, CT at
+// a time: the workgroup stages k, q, the decay (float, zero-padded to LPC * R rows), its v columns and sigmoid(beta) of CT
+// tokens in LDS - the next CT tokens' values are already in registers while these are computed - so a token's step reads
+// LDS only, and the only exchange on the state's dependency chain is the delta rule's S^T k; the read-outs' partial sums wait
+// in registers until the chunk's end and are exchanged together.  The state is read once before and written once after (a run
+// that starts its sequence starts from zeros).
+constexpr int SCAN_R = 16;        // rows of a column per lane
+constexpr int SCAN_CT = 16;       // tokens per staged chunk, at most
+constexpr int SCAN_PFK = 24;      // staged k / q / decay values per thread and chunk, at most
+constexpr int SCAN_PFV = 16;      // staged v values per thread and chunk, at most
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// sum over the lpc neighbouring lanes of a column (lpc a power of two); every one of them gets it
+__device__ __forceinline__ float column_sum(float v, int lpc) {
+    if (lpc >= 2) v = dpp_add<0xB1>(v);          // quad_perm [1, 0, 3, 2]
+    if (lpc >= 4) v = dpp_add<0x4E>(v);          // quad_perm [2, 3, 0, 1]
+    if (lpc >= 8) v = dpp_add<0x141>(v);         // row_half_mirror: the other quad of eight lanes
+    if (lpc >= 16) v = dpp_add<0x140>(v);        // row_mirror: the other half of sixteen lanes
+    if (lpc >= 32) v += __shfl_xor(v, 16, 64);
+    if (lpc >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+template <typename TQ, typename TB, bool DELTA>
+__global__ __launch_bounds__(512) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
+                                                             const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
+                                                             int64_t v_stride, const float* __restrict__ decay,
+                                                             const TB* __restrict__ beta, int64_t beta_stride,
+                                                             float* __restrict__ state, const int32_t* __restrict__ runs, int H,
+                                                             int QH, int dim, int vdim, int lpc_log, int CT, float q_scale) {
+    constexpr int R = SCAN_R;
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nthr >> 6;
+    const int lpc = 1 << lpc_log, cols = 64 >> lpc_log;
+    const int dimp_log = lpc_log + 4, DIMP = 1 << dimp_log, VB = nw * cols;       // (R = 16 = 2^4; nw and cols are powers of two)
+    const int vb_log = 31 - __clz(VB);
+    const int row_len = 3 * DIMP + ((VB + 4) & ~3);              // floats of one staged token: k | q | decay | v | beta, 16-byte rows
+    const int part = lane & (lpc - 1), cb = wave * cols + (lane >> lpc_log);
+    const int j = blockIdx.z * VB + cb;
     const bool col_ok = j < vdim;
     const int r0 = part * R;
     const int slot = runs[4 * blockIdx.x], first = runs[4 * blockIdx.x + 1], n = runs[4 * blockIdx.x + 2];
@@ -93,58 +123,107 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(float* __restrict__ 
 #pragma unroll
     for (int i = 0; i < R; ++i) S[i] = (!fresh && col_ok && r0 + i < dim) ? Sg[(size_t)(r0 + i) * vdim] : 0.f;
 
-    float kc[R], qc[R], gc[R], vc, bc = 0.f;
-    auto load = [&](int t, float (&kk)[R], float (&qq)[R], float (&gg)[R], float& vv, float& bb) {
-        const TQ* kr = k + (size_t)t * k_stride + (size_t)qh * dim;
-        const TQ* qr = q + (size_t)t * q_stride + (size_t)qh * dim;
-        const float* gr = decay + ((size_t)t * H + h) * (size_t)dim;
+    float pk[SCAN_PFK], pv[SCAN_PFV], pb = 0.f;
+    // requests the operands of tokens [c0, c0 + ct) of the run into registers
+    auto fetch = [&](int c0, int ct) {
+        const int nk = ct * 3 * DIMP, nv = ct * VB;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const bool ok = r0 + i < dim;
-            kk[i] = ok ? ld(kr, r0 + i) : 0.f;
-            qq[i] = ok ? ld(qr, r0 + i) : 0.f;
-            gg[i] = ok ? gr[r0 + i] : 0.f;
+        for (int i = 0; i < SCAN_PFK; ++i) {
+            const int idx = tid + i * nthr;
+            float val = 0.f;
+            if (idx < nk) {
+                const int seg = idx >> dimp_log, r = idx & (DIMP - 1), tt = seg / 3, which = seg - 3 * tt;
+                const size_t t = (size_t)(first + c0 + tt);
+                if (r < dim)
+                    val = which == 0 ? ld(k, t * k_stride + (size_t)qh * dim + r)
+                        : which == 1 ? ld(q, t * q_stride + (size_t)qh * dim + r)
+                                     : decay[(t * H + h) * (size_t)dim + r];
+            }
+            pk[i] = val;
         }
-        vv = col_ok ? ld(v, (size_t)t * v_stride + (size_t)h * vdim + j) : 0.f;
-        if (DELTA) bb = ld(beta, (size_t)t * beta_stride + h);
+#pragma unroll
+        for (int i = 0; i < SCAN_PFV; ++i) {
+            const int idx = tid + i * nthr;
+            float val = 0.f;
+            if (idx < nv) {
+                const int tt = idx >> vb_log, c = idx & (VB - 1), jj = blockIdx.z * VB + c;
+                if (jj < vdim) val = ld(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * vdim + jj);
+            }
+            pv[i] = val;
+        }
+        if (DELTA && tid < ct) pb = ld(beta, (size_t)(first + c0 + tid) * beta_stride + h);
     };
-    load(first, kc, qc, gc, vc, bc);
-    for (int t = first; t < first + n; ++t) {
-        float kn[R], qn[R], gn[R], vn = 0.f, bn = 0.f;
-        if (t + 1 < first + n) load(t + 1, kn, qn, gn, vn, bn);        // (wave-uniform)
-        float acc = 0.f;
-        if (DELTA) {
+    auto stage = [&](int ct) {
+        const int nk = ct * 3 * DIMP, nv = ct * VB;
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                S[i] *= gc[i];
-                acc += S[i] * kc[i];
-            }
-            for (int m = cols; m < 64; m <<= 1) acc += __shfl_xor(acc, m, 64);
-            const float u = (vc - acc) / (1.0f + expf(-bc));
-            acc = 0.f;
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                S[i] += kc[i] * u;
-                acc += S[i] * qc[i];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                S[i] = gc[i] * S[i] + kc[i] * vc;
-                acc += S[i] * qc[i];
+        for (int i = 0; i < SCAN_PFK; ++i) {
+            const int idx = tid + i * nthr;
+            if (idx < nk) {
+                const int tt = (idx >> dimp_log) / 3;
+                sm[tt * row_len + (idx - tt * 3 * DIMP)] = pk[i];
             }
         }
-        for (int m = cols; m < 64; m <<= 1) acc += __shfl_xor(acc, m, 64);
-        if (part == 0 && col_ok) o[((size_t)t * H + h) * (size_t)vdim + j] = acc * q_scale;
-        if (t + 1 < first + n) {
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                kc[i] = kn[i];
-                qc[i] = qn[i];
-                gc[i] = gn[i];
+        for (int i = 0; i < SCAN_PFV; ++i) {
+            const int idx = tid + i * nthr;
+            if (idx < nv) {
+                const int tt = idx >> vb_log;
+                sm[tt * row_len + 3 * DIMP + (idx & (VB - 1))] = pv[i];
             }
-            vc = vn;
-            bc = bn;
+        }
+        if (DELTA && tid < ct) sm[tid * row_len + 3 * DIMP + VB] = 1.0f / (1.0f + expf(-pb));
+    };
+
+    fetch(0, min(CT, n));
+    for (int c0 = 0; c0 < n; c0 += CT) {
+        const int ct = min(CT, n - c0);
+        __syncthreads();                                         // the previous chunk has been read by every wave
+        stage(ct);
+        __syncthreads();
+        if (c0 + CT < n) fetch(c0 + CT, min(CT, n - c0 - CT));   // in flight while this chunk is computed
+        float oacc[SCAN_CT];
+#pragma unroll
+        for (int tt = 0; tt < SCAN_CT; ++tt) {
+            oacc[tt] = 0.f;
+            if (tt >= ct) continue;                              // (uniform)
+            const float* row = sm + tt * row_len;
+            float kc[R], qc[R], gc[R];
+#pragma unroll
+            for (int i = 0; i < R; i += 4) {
+                const float4 a = *(const float4*)(row + r0 + i), b = *(const float4*)(row + DIMP + r0 + i),
+                             c = *(const float4*)(row + 2 * DIMP + r0 + i);
+                kc[i] = a.x; kc[i + 1] = a.y; kc[i + 2] = a.z; kc[i + 3] = a.w;
+                qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
+                gc[i] = c.x; gc[i + 1] = c.y; gc[i + 2] = c.z; gc[i + 3] = c.w;
+            }
+            const float vc = row[3 * DIMP + cb];
+            float acc = 0.f;
+            if (DELTA) {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    S[i] *= gc[i];
+                    acc += S[i] * kc[i];
+                }
+                const float u = (vc - column_sum(acc, lpc)) * row[3 * DIMP + VB];
+                acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    S[i] += kc[i] * u;
+                    acc += S[i] * qc[i];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    S[i] = gc[i] * S[i] + kc[i] * vc;
+                    acc += S[i] * qc[i];
+                }
+            }
+            oacc[tt] = acc;
+        }
+#pragma unroll
+        for (int tt = 0; tt < SCAN_CT; ++tt) {
+            const float sum = column_sum(oacc[tt], lpc);
+            if (tt < ct && part == 0 && col_ok) o[((size_t)(first + c0 + tt) * H + h) * (size_t)vdim + j] = sum * q_scale;
         }
     }
     if (col_ok) {
@@ -255,27 +334,38 @@ extern "C" int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, 
     return qsv_launch_status("qsv_conv_silu_unit");
 }
 
-extern "C" int qsv_recurrent_scan_rows(void) { return 16; }
-
 extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                                   int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
                                   int beta_dtype, float* state, const int32_t* runs, int n_runs, int heads, int qk_heads, int dim,
                                   int vdim, float q_scale, void* stream) {
-    constexpr int R = 16;
+    constexpr int R = SCAN_R;
     QSV_REQUIRE(o && q && k && v && decay && state && runs, "qsv_recurrent_scan: null argument");
     QSV_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dim > 0 && dim <= 64 * R && vdim > 0 && n_runs >= 0 &&
                     heads <= 65535,
                 "qsv_recurrent_scan: bad sizes (%d heads over %d, state %d x %d)", heads, qk_heads, dim, vdim);
     if (n_runs == 0) return QSV_OK;
-    int lpc = 1;
-    while (lpc * R < dim) lpc <<= 1;
-    const int cols = 64 / lpc;
-    const dim3 grid(n_runs, heads, (vdim + cols - 1) / cols), block(64);
+    int lpc = 1, lpc_log = 0;
+    while (lpc * R < dim) lpc <<= 1, ++lpc_log;
+    const int cols = 64 / lpc, DIMP = lpc * R;
+    const int waves_needed = (vdim + cols - 1) / cols;
+    // waves per workgroup: they share the staged k, q and decay.  Two, not more: a step is bound by instruction issue, and the
+    // launch's waves should spread over all SIMDs of the chip rather than stack up on the CUs of a few large workgroups
+    int nw = 1;
+    while (nw < 2 && nw < waves_needed) nw <<= 1;
+    const int VB = nw * cols, nthr = nw * 64;
+    int CT = SCAN_CT;                                            // tokens per staged chunk: what the prefetch registers and 48 KiB hold
+    while (CT > 1 && ((CT * 3 * DIMP + nthr - 1) / nthr > SCAN_PFK || (CT * VB + nthr - 1) / nthr > SCAN_PFV ||
+                      (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4 > 48 * 1024))
+        CT >>= 1;
+    QSV_REQUIRE((CT * 3 * DIMP + nthr - 1) / nthr <= SCAN_PFK && (CT * VB + nthr - 1) / nthr <= SCAN_PFV,
+                "qsv_recurrent_scan: a state of %d rows does not fit the staging registers", dim);
+    const size_t lds = (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4;
+    const dim3 grid(n_runs, heads, (vdim + VB - 1) / VB), block(nthr);
     QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
 #define QSV_SCAN(TQ, TB, DELTA)                                                                                              \
-    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, R>), grid, block, 0, (hipStream_t)stream, o, (const TQ*)q, q_stride, \
+    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA>), grid, block, lds, (hipStream_t)stream, o, (const TQ*)q, q_stride,  \
                        (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state, runs, heads,  \
-                       qk_heads, dim, vdim, lpc, q_scale)
+                       qk_heads, dim, vdim, lpc_log, CT, q_scale)
     if (beta) {
         if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_SCAN(float, float, true);
         else if (qkv_dtype == QSV_F32 && beta_dtype == QSV_BF16) QSV_SCAN(float, bf16_t, true);

@@ -7,7 +7,7 @@
 
 namespace {
 constexpr int NT = 256;
-constexpr int MAX_STREAMS = 8;
+constexpr int MAX_STREAMS = 16;
 
 template <typename T>
 __global__ __launch_bounds__(NT) void embed_streams_kernel(float* __restrict__ x, const T* __restrict__ table,
@@ -53,23 +53,29 @@ __global__ __launch_bounds__(NT) void hc_read_kernel(T* __restrict__ h, const fl
     }
 }
 
-// x[t, r] <- sum_s mix[s, r] x[t, s] + out[r] * y[t], all streams from the old ones
+// x[t, r] <- sum_s mix[s, r] x[t, s] + out[r] * y[t], all streams from the old ones; and, if asked for, the next sublayer's
+// input from the new streams in the same pass (no token shift there: that needs the previous token's NEW streams)
 template <typename T>
 __global__ __launch_bounds__(NT) void hc_write_kernel(float* __restrict__ x, const T* __restrict__ y, const float* __restrict__ mix,
-                                                      const float* __restrict__ w_out, int S, int D) {
+                                                      const float* __restrict__ w_out, int S, int D, T* __restrict__ h_next,
+                                                      const float* __restrict__ w_in_next, const T* __restrict__ nw,
+                                                      const T* __restrict__ nb, float alpha) {
     const size_t t = blockIdx.x;
     for (int i = threadIdx.x; i < D; i += NT) {
         float old[MAX_STREAMS];
 #pragma unroll
         for (int s = 0; s < MAX_STREAMS; ++s) old[s] = s < S ? x[(t * S + s) * D + i] : 0.f;
         const float yv = ld(y, t * D + i);
+        float u = 0.f;
         for (int r = 0; r < S; ++r) {
             float a = w_out[r] * yv;
 #pragma unroll
             for (int s = 0; s < MAX_STREAMS; ++s)
                 if (s < S) a += mix[s * S + r] * old[s];
             x[(t * S + r) * D + i] = a;
+            if (h_next) u += w_in_next[r] * a;
         }
+        if (h_next) st(h_next, t * D + i, tanhf(alpha * u) * ld(nw, i) + ld(nb, i));
     }
 }
 
@@ -137,14 +143,15 @@ extern "C" int qsv_hc_read(void* h, const float* x, const float* w_in, const voi
     return qsv_launch_status("qsv_hc_read");
 }
 
-extern "C" int qsv_hc_write(float* x, const void* y, const float* mix, const float* w_out, int n, int streams, int D, int dtype,
-                            void* stream) {
+extern "C" int qsv_hc_write(float* x, const void* y, const float* mix, const float* w_out, int n, int streams, int D, void* h_next,
+                            const float* w_in_next, const void* norm_w, const void* norm_b, float alpha, int dtype, void* stream) {
     QSV_REQUIRE(x && y && mix && w_out && n >= 0 && D > 0, "qsv_hc_write: bad arguments");
+    QSV_REQUIRE(!h_next || (w_in_next && norm_w && norm_b), "qsv_hc_write: the next sublayer's input without its weights");
     QSV_REQUIRE(streams > 0 && streams <= MAX_STREAMS, "qsv_hc_write: %d streams (at most %d)", streams, MAX_STREAMS);
     if (n == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_hc_write",
                  hipLaunchKernelGGL(hc_write_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (const T*)y, mix, w_out,
-                                    streams, D));
+                                    streams, D, (T*)h_next, w_in_next, (const T*)norm_w, (const T*)norm_b, alpha));
     return qsv_launch_status("qsv_hc_write");
 }
 

@@ -93,10 +93,10 @@ class HipOps:
 
     attention_split_target = 512        # workgroups a launch of the matrix-core attention should at least have
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0):
         """batch: the step's StepBatch (block table, sequence slot and position per token, work tiles).  variant: 0 = the
         matrix-core kernel where it takes the sizes, 1 = always the wave kernel.  key_splits: None = chosen from the number
-        of workgroups and the context."""
+        of workgroups and the context.  q_first: the caller's promise that every query is zero before that element."""
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
@@ -118,7 +118,7 @@ class HipOps:
                                                         block_table.stride(0), pos.data_ptr(), tiles.data_ptr(), tiles.size(0),
                                                         int(window or 0), H, rank, R, page, splits,
                                                         0 if po is None else po.data_ptr(), 0 if pm is None else pm.data_ptr(), T,
-                                                        self._s()), "latent_attention_mfma")
+                                                        int(q_first), self._s()), "latent_attention_mfma")
             return out
         self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
@@ -158,13 +158,20 @@ class HipOps:
                                       T, S, D, self.code, self._s()), "hc_read")
         return h
 
-    def hc_write(self, x, y, w_mix, w_out):
+    def hc_write(self, x, y, w_mix, w_out, then_read=None):
+        """All streams rewritten in place from the sublayer's output y.  then_read = (w_in, norm) of the NEXT sublayer, if it
+        reads without a token shift: its input comes out of the same pass -> h [T, D] (else None)."""
         T, S, D = x.shape
         self._need(x, y, w_mix, w_out)
         assert y.shape == (T, D) and y.dtype == self.dtype and w_mix.dtype == torch.float32 and w_mix.shape == (S, S)
-        self.check(self.L.qsv_hc_write(x.data_ptr(), y.data_ptr(), w_mix.data_ptr(), w_out.data_ptr(), T, S, D, self.code, self._s()),
-                   "hc_write")
-        return x
+        h, nxt = None, [0, 0, 0, 0, 0.0]
+        if then_read is not None:
+            w_in, (w, b, alpha) = then_read
+            h = torch.empty((T, D), dtype=self.dtype, device=x.device)
+            nxt = [h.data_ptr(), w_in.data_ptr(), w.data_ptr(), b.data_ptr(), float(alpha)]
+        self.check(self.L.qsv_hc_write(x.data_ptr(), y.data_ptr(), w_mix.data_ptr(), w_out.data_ptr(), T, S, D, *nxt, self.code,
+                                       self._s()), "hc_write")
+        return h
 
     def dyt_sum_rows(self, x, rows, norm):
         w, b, alpha = norm
@@ -332,11 +339,11 @@ class HipOps:
                                           self._s()), "moe_combine")
         return y
 
-    def _moe_experts_sorted(self, h, up, down, idx, wt, a=1):
-        """a = 2 (gated units): the first product leaves both halves of every unit ([n, 2 ff]), `glu` folds them."""
+    def _moe_experts_sorted(self, h, up, down, idx, wt, code=1):
+        """code = 2 (gated units): the first product leaves both halves of every unit ([n, 2 ff]), `glu` folds them."""
         T, D = h.shape
         E, rows, K = up.size(0), up.size(1), idx.size(1)
-        ff = rows // 2 if a == 2 else rows
+        ff = rows // 2 if code == 2 else rows
         n = T * K
         flat = idx.reshape(-1)
         order = torch.argsort(flat, stable=True)                       # sorted slot -> slot (t K + k)
@@ -355,8 +362,8 @@ class HipOps:
             tls = [torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device) for lo in range(0, len(tiles), 65535)]
             for tl in tls:
                 self.check(self.L.qsv_grouped_gemm(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), tl.data_ptr(),
-                                                   tl.size(0), rows, D, 1 if a == 1 else 0, self._s()), "grouped_gemm(up)")
-            if a == 2:
+                                                   tl.size(0), rows, D, 1 if code == 1 else 0, self._s()), "grouped_gemm(up)")
+            if code == 2:
                 act = self.glu(act)
             for tl in tls:
                 self.check(self.L.qsv_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), tl.data_ptr(),
@@ -375,7 +382,7 @@ class HipOps:
             if c:
                 torch.matmul(xs[at:at + c], up[e].t(), out=act[at:at + c])
             at += c
-        if a == 2:
+        if code == 2:
             act = self.glu(act)
         else:
             self.check(self.L.qsv_relu_sq(act.data_ptr(), act.numel(), self.code, self._s()), "relu_sq")
@@ -448,7 +455,7 @@ class TorchOps:
         qr = _rotate(q.view(T, heads, dim + rot_dim)[..., dim:].float(), rope, pos, rot_n)
         return (torch.cat([q_abs.transpose(0, 1).float(), qr], dim=-1) * scale).contiguous()
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0):
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
@@ -484,9 +491,9 @@ class TorchOps:
             prev[wr] = n[first + cnt - 1]
         return (n + (before - n) * shift.float()).to(self.dtype)
 
-    def hc_write(self, x, y, w_mix, w_out):
+    def hc_write(self, x, y, w_mix, w_out, then_read=None):
         x.copy_(torch.einsum("sr,tsd->trd", w_mix, x) + w_out[None, :, None] * y.float()[:, None, :])
-        return x
+        return None if then_read is None else self.hc_read(x, then_read[0], then_read[1])
 
     def dyt_sum_rows(self, x, rows, norm):
         w, b, alpha = norm

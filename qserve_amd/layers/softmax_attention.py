@@ -38,11 +38,11 @@ class RotatedValueAttention:
                                 self.rope_k.reserve(n), self.rope_v.reserve(n), self.scale, pool, batch)
         per = H // G
         if G == 1:
-            o = ops.latent_attention(qf, pool[0], batch, None, self.vdim, self.page)
+            o = ops.latent_attention(qf, pool[0], batch, None, self.vdim, self.page, q_first=self.vdim)
         else:
             o = torch.empty((T, H, self.vdim), dtype=h.dtype, device=h.device)
             for g in range(G):
                 o[:, g * per:(g + 1) * per] = ops.latent_attention(qf[:, g * per:(g + 1) * per].contiguous(), pool[g], batch, None,
-                                                                   self.vdim, self.page)
+                                                                   self.vdim, self.page, q_first=self.vdim)
         ops.rotate_heads(o, self.rope_v.table, batch.pos, -1.0)
         return linear(o.view(T, H * self.vdim), self.w_o)

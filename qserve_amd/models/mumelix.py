@@ -134,10 +134,12 @@ class Mumelix:
             p0, p1, s0, s1 = self.run_slices[run]
             w_in, w_mix, w_out = L["hc1"]
             h = ops.hc_read(x, w_in, L["norm1"], L["shift"], batch, states[s0])
-            ops.hc_write(x, L["mixer"](h, batch, pools[p0:p1], states[s0 + 1:s1]), w_mix, w_out)
-            if L["ff"] is not None:
-                w_in, w_mix, w_out = L["hc2"]
-                ops.hc_write(x, L["ff"](ops.hc_read(x, w_in, L["norm2"])), w_mix, w_out)
+            y = L["mixer"](h, batch, pools[p0:p1], states[s0 + 1:s1])
+            if L["ff"] is None:
+                ops.hc_write(x, y, w_mix, w_out)
+            else:                                               # the feed-forward's input comes out of the mixer's stream rewrite
+                h = ops.hc_write(x, y, w_mix, w_out, then_read=(L["hc2"][0], L["norm2"]))
+                ops.hc_write(x, L["ff"](h), L["hc2"][1], L["hc2"][2])
             if tap is not None:
                 tap(run, x.sum(1))
         return x

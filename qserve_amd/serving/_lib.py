@@ -20,7 +20,7 @@ SIGNATURES = {
     "qsv_latent_attention": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "qsv_latent_attention_tile_tokens": (_i, [_i]),
     "qsv_latent_attention_mfma_ok": (_i, [_i, _i, _i]),
-    "qsv_latent_attention_mfma": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
+    "qsv_latent_attention_mfma": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "qsv_sigmoid_gate": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp]),
     "qsv_moe_route": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "qsv_moe_up": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
@@ -34,7 +34,7 @@ SIGNATURES = {
     "qsv_moe_down": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "qsv_embed_streams": (_i, [_vp, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
     "qsv_hc_read": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
-    "qsv_hc_write": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "qsv_hc_write": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _vp]),
     "qsv_dyt_sum_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
     "qsv_rms_pair_mean": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _vp]),
     "qsv_glu": (_i, [_vp, _vp, _i, _i, _i, _vp]),

@@ -1,6 +1,7 @@
-"""Throughput of a served design at layer sizes of real models, beside the W4A8KV4 Llama engine at equal size.
+"""Throughput of a served design at layer sizes of real models, beside the closest existing model at equal size.
 
-    python bench.py --design vekalorn [--design-sizes w2048,w4096] [--steps K] [--warmup W]
+    python bench.py --design vekalorn [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside the W4A8KV4 Llama engine
+    python bench.py --design mumelix  [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside Vekalorn
 
 Per size (random weights, 4 layers, vocabulary 32000): prompt phase = 8 prompts x 1024 tokens in one step through
 Engine.execute; decoding = 64 sequences at context 1024, one token each per step.  Beside them the Llama-style W4A8KV4
@@ -73,12 +74,23 @@ def random_weights(cfg, dev, seed=0):
 class OpTimer:
     """HIP events around every call of the ops object's methods and of the vendor products (one step at a time)."""
     NAMES = ("embed", "add_layer_norm", "layer_norm_rows", "latent_prep", "latent_query", "latent_attention", "sigmoid_gate",
-             "moe_route", "moe_experts")
+             "moe_route", "moe_experts", "embed_streams", "hc_read", "hc_write", "dyt_sum_rows", "rms_pair_mean", "glu",
+             "attention_prep", "rotate_heads", "decay", "conv_silu_unit", "recurrent_scan", "head_rms_gate")
 
     def __init__(self, ops):
         self.ops, self.events, self.calls, self.on = ops, [], [], False
         for n in self.NAMES:
             setattr(ops, n, self._wrap(n, getattr(ops, n)))
+        from ..layers import ops as ops_module                # the vendor products, as the layers call them
+        for mod in self._linear_users():
+            mod.linear = self._wrap("linear", ops_module.linear)
+
+    @staticmethod
+    def _linear_users():
+        import importlib
+        return [importlib.import_module("qserve_amd." + m) for m in
+                ("layers.latent_attention", "layers.moe", "layers.recurrent", "layers.softmax_attention", "models.vekalorn",
+                 "models.mumelix")]
 
     def _wrap(self, name, fn):
         def timed(*a, **k):
@@ -246,6 +258,150 @@ def bench_llama(name, s, dev, steps, warmup, helpers):
                 roofline=dict(decode_gemm_frac_hbm=sum(r["bytes"] for r in gemm) / sum(r["us"] for r in gemm) / 1e3 / HBM_PEAK_GBS))
 
 
+# ---- Mumelix ----------------------------------------------------------------------------------------------------------------
+FP32_VALU_PEAK_TFLOPS = 157.0
+MUMELIX = {
+    "w2048": dict(g_heads=16, g_dim=64, g_vdim=128, a_heads=16, a_kv=4, a_dim=128, a_vdim=128, rot=64, d_heads=16, d_kv=4,
+                  d_dim=64, d_vdim=128, taps=4, low=64, streams=2),
+    "w4096": dict(g_heads=32, g_dim=64, g_vdim=128, a_heads=32, a_kv=8, a_dim=128, a_vdim=128, rot=64, d_heads=32, d_kv=8,
+                  d_dim=64, d_vdim=128, taps=4, low=128, streams=2),
+}
+
+
+def mumelix_config(s, m):
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"]}, "router": {"experts": s["experts"], "top": s["top"]}}
+    g = {"type": "gla", "mlp": mlp, "mixer": {"heads": m["g_heads"], "dim": m["g_dim"], "vdim": m["g_vdim"], "tau": 16.0}}
+    rot = {"base": 500000.0, "dims": m["rot"], "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    p = {"type": "parallel", "mlp": mlp,
+         "mixer": {"left": {"heads": m["a_heads"], "kv_heads": m["a_kv"], "dim": m["a_dim"], "vdim": m["a_vdim"], "rot": rot,
+                            "scale": 1.0 / math.sqrt(m["a_dim"])},
+                   "right": {"heads": m["d_heads"], "kv_heads": m["d_kv"], "dim": m["d_dim"], "vdim": m["d_vdim"], "conv": m["taps"]}}}
+    return {"architecture": "Mumelix", "width": s["width"], "vocab": VOCAB, "streams": m["streams"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-5}, "layers": [g, p, g, p][:LAYERS]}
+
+
+def mumelix_weights(cfg, m, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    D, V, S, r = cfg["width"], cfg["vocab"], cfg["streams"], m["low"]
+
+    def mat(o, i, s=1.0):
+        return (torch.randn((o, i), device=dev, generator=g) * (s / math.sqrt(i))).bfloat16()
+
+    def vec(n, mean=1.0, s=0.1):
+        return (mean + s * torch.randn((n,), device=dev, generator=g)).bfloat16()
+
+    W = {"embed": torch.randn((V, D), device=dev, generator=g).bfloat16(), "head": mat(V, D)}
+
+    def norm(name):
+        W[name], W[name + ".b"], W[name + ".alpha"] = vec(D), vec(D, 0.0), torch.tensor(0.7).bfloat16()
+
+    norm("final.norm")
+    for i, L in enumerate(cfg["layers"]):
+        p, x = f"l{i}.", L["mixer"]
+        norm(p + "norm1"), norm(p + "norm2")
+        W[p + "shift"] = vec(D, 0.5, 0.2)
+        for q in (1, 2):
+            W[p + f"hc{q}.in"], W[p + f"hc{q}.out"] = vec(S, 1.0 / S), vec(S, 1.0)
+            W[p + f"hc{q}.mix"] = (torch.eye(S, device=dev) * 0.9 + 0.05).bfloat16()
+        if L["type"] == "gla":
+            H, d, dv = x["heads"], x["dim"], x["vdim"]
+            W.update({p + "mix.q": mat(H * d, D), p + "mix.k": mat(H * d, D), p + "mix.v": mat(H * dv, D), p + "mix.g": mat(H * dv, D),
+                      p + "mix.o": mat(D, H * dv), p + "mix.norm": vec(dv), p + "mix.a1": mat(r, D), p + "mix.a2": mat(H * d, r),
+                      p + "mix.a2.b": vec(H * d, 3.0, 1.0)})
+        else:
+            a, b = x["left"], x["right"]
+            q = p + "mix.left."
+            W.update({q + "q": mat(a["heads"] * a["dim"], D), q + "k": mat(a["kv_heads"] * a["dim"], D),
+                      q + "v": mat(a["kv_heads"] * a["vdim"], D), q + "o": mat(D, a["heads"] * a["vdim"]), q + "out": vec(D)})
+            q = p + "mix.right."
+            H, G, d, dv, taps = b["heads"], b["kv_heads"], b["dim"], b["vdim"], b["conv"]
+            W.update({q + "q": mat(G * d, D), q + "k": mat(G * d, D), q + "v": mat(H * dv, D), q + "q.conv": mat(G * d, taps),
+                      q + "k.conv": mat(G * d, taps), q + "v.conv": mat(H * dv, taps), q + "b": mat(H, D), q + "A_log": vec(H, -1.0, 0.5),
+                      q + "norm": vec(dv), q + "a1": mat(r, D), q + "a2": mat(H * d, r), q + "dt_bias": vec(H * d, -1.0, 1.0),
+                      q + "g1": mat(r, D), q + "g2": mat(H * dv, r), q + "o": mat(D, H * dv), q + "out": vec(D)})
+        E, ff = L["mlp"]["router"]["experts"], L["mlp"]["expert"]["ff"]
+        for e in range(E):
+            W[f"{p}mlp.e{e}.gate"], W[f"{p}mlp.e{e}.up"], W[f"{p}mlp.e{e}.down"] = mat(ff, D), mat(ff, D), mat(D, ff)
+        W[p + "mlp.router"], W[p + "mlp.router.b"] = mat(E, D, 3.0), vec(E, 0.0, 0.5)
+    return W
+
+
+def bench_mumelix(name, s, dev, steps, warmup):
+    from ..models.mumelix import Mumelix
+    from .engine import Engine
+    m = MUMELIX[name]
+    cfg = mumelix_config(s, m)
+    NB, L, BP = 64, 1024, 8
+    eng = Engine(Mumelix, cfg, mumelix_weights(cfg, m, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 384), max_seqs=NB)
+    timer = OpTimer(eng.ops)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, VOCAB, (L,), generator=g).tolist() for _ in range(NB)]
+    slots = [eng.open_sequence() for _ in range(NB)]
+    pre_ms, ops_pre, rep_pre = [], None, {}
+    for i in range(0, NB, BP):
+        items = [(slots[j], prompts[j]) for j in range(i, i + BP)]
+        want = [k * L + L - 1 for k in range(BP)]
+        if i == BP:                                          # one step with events around every launch
+            ops_pre, _ = timer.step(lambda: eng.execute(items, want))
+            rep_pre = {k: timer.replay(k, 3) for k in ("latent_attention", "hc_read", "hc_write")}
+            continue
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.execute(items, want)
+        torch.cuda.synchronize()
+        if i > 0:
+            pre_ms.append((time.perf_counter() - t0) * 1e3)
+    pre = sorted(pre_ms)[len(pre_ms) // 2]
+    nxt = [[int(torch.randint(0, VOCAB, (1,), generator=g))] for _ in range(NB)]
+    want = list(range(NB))
+
+    def decode():
+        eng.execute([(slots[j], nxt[j]) for j in range(NB)], want)
+
+    dec_eager = timed(decode, steps, warmup)
+    ops_dec, dec_events_ms = timer.step(decode)
+    rep_dec = {k: timer.replay(k, 20) for k in ("latent_attention", "moe_experts", "hc_read", "hc_write")}
+    eng.decode_graphs = True
+    dec = timed(decode, steps, warmup)
+    graph_ok = any(v is not False for v in eng._graphs.values()) and bool(eng._graphs)
+    ctx = eng.cache.length[slots[0]]
+    T, D, S = BP * L, s["width"], m["streams"]
+    n_att = sum(1 for x in cfg["layers"] if x["type"] == "parallel")
+    n_gla = LAYERS - n_att
+    R = m["a_dim"] + m["a_vdim"]
+    # attention: useful work = q.k over dim and p.v over vdim (the kernel also multiplies the query's zero half)
+    att_flops = n_att * BP * sum(p + 1 for p in range(L)) * m["a_heads"] * (m["a_dim"] + m["a_vdim"]) * 2.0
+    att_pre = att_flops / (rep_pre["latent_attention"] * 1e-3) / 1e12
+    att_bytes = n_att * NB * ctx * m["a_kv"] * R * 2.0
+    att_dec = att_bytes / (rep_dec["latent_attention"] * 1e-3) / 1e9
+    # recurrences: 5 (gated linear attention) / 7 (delta rule) float operations per state element and token; decoding moves the state twice
+    el = n_gla * m["g_heads"] * m["g_dim"] * m["g_vdim"], n_att * m["d_heads"] * m["d_dim"] * m["d_vdim"]
+    scan_pre = T * (5.0 * el[0] + 7.0 * el[1]) / (ops_pre["recurrent_scan"] * 1e-3) / 1e12
+    scan_dec = NB * (el[0] + el[1]) * 4.0 * 2 / (ops_dec["recurrent_scan"] * 1e-3) / 1e9
+    moe_flops = LAYERS * T * s["top"] * 3 * 2.0 * s["ff"] * D
+    moe_pre = moe_flops / (ops_pre["moe_experts"] * 1e-3) / 1e12
+    moe_bytes = LAYERS * min(s["experts"], NB * s["top"]) * 3 * s["ff"] * D * 2.0
+    moe_dec = moe_bytes / (rep_dec["moe_experts"] * 1e-3) / 1e9
+    # stream kernels: read S streams per sublayer, rewrite S streams (read + write) per sublayer, float
+    hc_bytes = LAYERS * 2 * (S * D * 4.0 + D * 2.0) + LAYERS * 2 * (2 * S * D * 4.0 + D * 2.0)
+    hc_pre = T * hc_bytes / ((rep_pre["hc_read"] + rep_pre["hc_write"]) * 1e-3) / 1e9
+    out = dict(model=f"Mumelix-{name}", sizes=m, prefill_tokens_per_s=T / pre * 1e3, prefill_ms=pre, decode_tokens_per_s=NB / dec * 1e3,
+               decode_ms=dec, decode_from_hipgraph=graph_ok, decode_ms_eager=dec_eager, decode_ms_gpu_events=dec_events_ms, context=ctx,
+               prefill_ops_ms=ops_pre, decode_ops_ms=ops_dec, prefill_kernels_ms=rep_pre, decode_kernels_ms=rep_dec,
+               roofline=dict(prefill_attention_tflops=att_pre, prefill_attention_frac_bf16_peak=att_pre / BF16_PEAK_TFLOPS,
+                             decode_attention_gbs=att_dec, decode_attention_frac_hbm=att_dec / HBM_PEAK_GBS,
+                             prefill_experts_tflops=moe_pre, prefill_experts_frac_bf16_peak=moe_pre / BF16_PEAK_TFLOPS,
+                             decode_experts_gbs=moe_dec, decode_experts_frac_hbm=moe_dec / HBM_PEAK_GBS,
+                             prefill_recurrence_tflops=scan_pre, prefill_recurrence_frac_fp32_valu_peak=scan_pre / FP32_VALU_PEAK_TFLOPS,
+                             decode_recurrence_gbs=scan_dec, decode_recurrence_frac_hbm=scan_dec / HBM_PEAK_GBS,
+                             prefill_stream_kernels_gbs=hc_pre, prefill_stream_kernels_frac_hbm=hc_pre / HBM_PEAK_GBS))
+    for sl in slots:
+        eng.close_sequence(sl)
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
 def main(args, helpers):
     dev = "cuda:0"
     torch.cuda.set_device(0)
@@ -255,10 +411,16 @@ def main(args, helpers):
         build.build(verbose=False)
     steps, warmup = min(args.steps, 32), min(args.warmup, 8)
     for name in args.design_sizes.split(","):
+        if args.design == "mumelix" and name not in MUMELIX:      # (sizes that differ in a Vekalorn-only constant)
+            continue
         s = SIZES[name]
         line = {"design": args.design, "size": name, "sizes": s, "layers": LAYERS, "vocab": VOCAB, "dtype": "bf16",
                 "data": "synthetic", "workload": "prefill 8 x 1024 tokens in one step; decode 64 sequences at context 1024"}
-        line["vekalorn"] = bench_vekalorn(name, s, dev, steps, warmup)
-        line["llama_w4a8"] = bench_llama(name, s, dev, steps, warmup, helpers)
+        if args.design == "mumelix":
+            line["mumelix"] = bench_mumelix(name, s, dev, steps, warmup)
+            line["vekalorn"] = bench_vekalorn(name, s, dev, steps, warmup)
+        else:
+            line["vekalorn"] = bench_vekalorn(name, s, dev, steps, warmup)
+            line["llama_w4a8"] = bench_llama(name, s, dev, steps, warmup, helpers)
         print(json.dumps(line), flush=True)
     return 0

@@ -37,9 +37,10 @@ class StepBatch:
     _runs: torch.Tensor = None
 
     def runs(self):
-        """int32 [n_runs, 4] = (sequence slot, first flat token index, tokens, position of the first token), on the device."""
+        """int32 [n_runs, 4] = (sequence slot, first flat token index, tokens, position of the first token), on the device.
+        The engine's layout brings it along with the other metadata; a batch made by hand gets it here (one synchronisation)."""
         if self._runs is None:
-            pos = self.pos.tolist() if self.pos is not None else None
+            pos = self.pos.tolist()
             rows = [(slot, first, n, pos[first]) for slot, first, n in self.items]
             self._runs = torch.tensor(rows, dtype=torch.int32).reshape(-1, 4).to(self.pos.device)
         return self._runs
@@ -127,11 +128,13 @@ class Engine:
 
     def _to_device(self, meta, rows, runs):
         dev = self.device
-        max_pos = int(meta[2].max())
-        meta = meta.to(dev)                    # (one host tensor, one copy)
+        max_pos, T = int(meta[2].max()), meta.size(1)
+        runs4 = torch.tensor([(s, first, n, int(meta[2, first])) for s, first, n in runs], dtype=torch.int32)
+        flat = torch.cat([meta.reshape(-1), runs4.reshape(-1)]).to(dev)      # (one host tensor, one copy)
+        meta = flat[:6 * T].view(6, T)
         return StepBatch(tokens=meta[0], seq=meta[1], pos=meta[2], slot=torch.tensor(rows, dtype=torch.int64).to(dev),
-                         block_table=self.cache.block_table(), max_pos=max_pos, n_tokens=meta.size(1), items=runs,
-                         run_off=meta[3], state_rd=meta[4], state_wr=meta[5])
+                         block_table=self.cache.block_table(), max_pos=max_pos, n_tokens=T, items=runs,
+                         run_off=meta[3], state_rd=meta[4], state_wr=meta[5], _runs=flat[6 * T:].view(-1, 4))
 
     @torch.no_grad()
     def execute(self, items, want):

@@ -571,3 +571,42 @@ def test_decode_steps_from_a_graph_match_eager_steps(dtype, std):
         assert_close(got[1][k], got[0][k], tol, f"graph against eager, sequence {k}")
         if dtype == "float32":
             assert_close(got[1][k], ref[k][:got[0][k].shape[0]], F32_TOL, f"graph against the oracle, sequence {k}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("E,top,ff,D,T", [(6, 3, 24, 40, 33), (16, 4, 136, 264, 64), (8, 2, 128, 192, 300), (3, 1, 64, 64, 70),
+                                          (4, 4, 704, 1024, 150), (8, 8, 520, 2056, 3)])
+def test_gated_expert_forms_agree_in_bfloat16(E, top, ff, D, T):
+    """Per-token kernels, expert-major kernels, the grouped matrix-core kernel (widths that are multiples of its K step) and
+    expert-sorted vendor products on the same bfloat16 inputs, against the float64 sum over the chosen gated experts."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from qserve_amd.layers.moe import _interleave
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(E * 100 + T)
+    h = torch.randn(T, D, generator=g).bfloat16()
+    gate = (torch.randn(E, ff, D, generator=g) / math.sqrt(D)).bfloat16()
+    up = (torch.randn(E, ff, D, generator=g) / math.sqrt(D)).bfloat16()
+    down = (torch.randn(E, D, ff, generator=g) / math.sqrt(ff)).bfloat16()
+    idx = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).int()
+    if T > 4:
+        idx[:, 0] = idx[0, 0]                                            # one expert shared by many tokens, some experts unused
+    wt = torch.rand(T, top, generator=g)
+    ref = torch.zeros(T, D, dtype=torch.float64)
+    for t in range(T):
+        for k in range(top):
+            e = int(idx[t, k])
+            a = P.silu(gate[e].double() @ h[t].double()) * (up[e].double() @ h[t].double())
+            ref[t] += wt[t, k].double() * (down[e].double() @ a)
+    forms = {"per-token": dict(moe_token_slots=10 ** 9, moe_sorted_above=10 ** 9),
+             "expert-major": dict(moe_token_slots=0, moe_expert_major_slots=10 ** 9),
+             "expert-sorted, grouped kernel": dict(moe_token_slots=10 ** 9, moe_expert_major_slots=0, moe_sorted_above=0),
+             "expert-sorted, vendor products": dict(moe_token_slots=10 ** 9, moe_expert_major_slots=0, moe_sorted_above=0,
+                                                    moe_grouped_kernel=False)}
+    w_in = _interleave(gate, up).to(dev)
+    for name, knobs in forms.items():
+        o = make_ops("hip", torch.bfloat16, dev)
+        for k, v in knobs.items():
+            setattr(o, k, v)
+        y = o.moe_experts(h.to(dev), w_in, down.to(dev), idx.to(dev), wt.to(dev), act="swiglu").double().cpu()
+        assert_close(y, ref, 2e-2, f"{name} form")
