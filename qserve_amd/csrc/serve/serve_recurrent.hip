@@ -97,7 +97,15 @@ __device__ __forceinline__ float column_sum(float v, int lpc) {
     return v;
 }
 
-template <typename TQ, typename TB, bool DELTA>
+__device__ __forceinline__ float4 ld4(const float* p, size_t i) { return *(const float4*)(p + i); }
+__device__ __forceinline__ float4 ld4(const bf16_t* p, size_t i) {
+    const uint2 u = *(const uint2*)(p + i);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                       __uint_as_float(u.y & 0xffff0000u));
+}
+
+// VEC: dim, vdim, the row strides and the operands' addresses are multiples of four elements - staged four at a time
+template <typename TQ, typename TB, bool DELTA, bool VEC>
 __global__ __launch_bounds__(512) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
                                                              const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
                                                              int64_t v_stride, const float* __restrict__ decay,
@@ -127,48 +135,94 @@ __global__ __launch_bounds__(512) void recurrent_scan_kernel(float* __restrict__
     // requests the operands of tokens [c0, c0 + ct) of the run into registers
     auto fetch = [&](int c0, int ct) {
         const int nk = ct * 3 * DIMP, nv = ct * VB;
+        if (VEC) {
 #pragma unroll
-        for (int i = 0; i < SCAN_PFK; ++i) {
-            const int idx = tid + i * nthr;
-            float val = 0.f;
-            if (idx < nk) {
-                const int seg = idx >> dimp_log, r = idx & (DIMP - 1), tt = seg / 3, which = seg - 3 * tt;
-                const size_t t = (size_t)(first + c0 + tt);
-                if (r < dim)
-                    val = which == 0 ? ld(k, t * k_stride + (size_t)qh * dim + r)
-                        : which == 1 ? ld(q, t * q_stride + (size_t)qh * dim + r)
-                                     : decay[(t * H + h) * (size_t)dim + r];
+            for (int i = 0; i < SCAN_PFK / 4; ++i) {
+                const int idx = (tid + i * nthr) * 4;
+                float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < nk) {
+                    const int seg = idx >> dimp_log, r = idx & (DIMP - 1), tt = seg / 3, which = seg - 3 * tt;
+                    const size_t t = (size_t)(first + c0 + tt);
+                    if (r < dim)
+                        val = which == 0 ? ld4(k, t * k_stride + (size_t)qh * dim + r)
+                            : which == 1 ? ld4(q, t * q_stride + (size_t)qh * dim + r)
+                                         : ld4(decay, (t * H + h) * (size_t)dim + r);
+                }
+                pk[4 * i] = val.x; pk[4 * i + 1] = val.y; pk[4 * i + 2] = val.z; pk[4 * i + 3] = val.w;
             }
-            pk[i] = val;
-        }
 #pragma unroll
-        for (int i = 0; i < SCAN_PFV; ++i) {
-            const int idx = tid + i * nthr;
-            float val = 0.f;
-            if (idx < nv) {
-                const int tt = idx >> vb_log, c = idx & (VB - 1), jj = blockIdx.z * VB + c;
-                if (jj < vdim) val = ld(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * vdim + jj);
+            for (int i = 0; i < SCAN_PFV / 4; ++i) {
+                const int idx = (tid + i * nthr) * 4;
+                float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < nv) {
+                    const int tt = idx >> vb_log, c = idx & (VB - 1), jj = blockIdx.z * VB + c;
+                    if (jj < vdim) val = ld4(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * vdim + jj);
+                }
+                pv[4 * i] = val.x; pv[4 * i + 1] = val.y; pv[4 * i + 2] = val.z; pv[4 * i + 3] = val.w;
             }
-            pv[i] = val;
+        } else {
+#pragma unroll
+            for (int i = 0; i < SCAN_PFK; ++i) {
+                const int idx = tid + i * nthr;
+                float val = 0.f;
+                if (idx < nk) {
+                    const int seg = idx >> dimp_log, r = idx & (DIMP - 1), tt = seg / 3, which = seg - 3 * tt;
+                    const size_t t = (size_t)(first + c0 + tt);
+                    if (r < dim)
+                        val = which == 0 ? ld(k, t * k_stride + (size_t)qh * dim + r)
+                            : which == 1 ? ld(q, t * q_stride + (size_t)qh * dim + r)
+                                         : decay[(t * H + h) * (size_t)dim + r];
+                }
+                pk[i] = val;
+            }
+#pragma unroll
+            for (int i = 0; i < SCAN_PFV; ++i) {
+                const int idx = tid + i * nthr;
+                float val = 0.f;
+                if (idx < nv) {
+                    const int tt = idx >> vb_log, c = idx & (VB - 1), jj = blockIdx.z * VB + c;
+                    if (jj < vdim) val = ld(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * vdim + jj);
+                }
+                pv[i] = val;
+            }
         }
         if (DELTA && tid < ct) pb = ld(beta, (size_t)(first + c0 + tid) * beta_stride + h);
     };
     auto stage = [&](int ct) {
         const int nk = ct * 3 * DIMP, nv = ct * VB;
+        if (VEC) {
 #pragma unroll
-        for (int i = 0; i < SCAN_PFK; ++i) {
-            const int idx = tid + i * nthr;
-            if (idx < nk) {
-                const int tt = (idx >> dimp_log) / 3;
-                sm[tt * row_len + (idx - tt * 3 * DIMP)] = pk[i];
+            for (int i = 0; i < SCAN_PFK / 4; ++i) {
+                const int idx = (tid + i * nthr) * 4;
+                if (idx < nk) {
+                    const int tt = (idx >> dimp_log) / 3;
+                    *(float4*)(sm + tt * row_len + (idx - tt * 3 * DIMP)) = make_float4(pk[4 * i], pk[4 * i + 1], pk[4 * i + 2], pk[4 * i + 3]);
+                }
             }
-        }
 #pragma unroll
-        for (int i = 0; i < SCAN_PFV; ++i) {
-            const int idx = tid + i * nthr;
-            if (idx < nv) {
-                const int tt = idx >> vb_log;
-                sm[tt * row_len + 3 * DIMP + (idx & (VB - 1))] = pv[i];
+            for (int i = 0; i < SCAN_PFV / 4; ++i) {
+                const int idx = (tid + i * nthr) * 4;
+                if (idx < nv) {
+                    const int tt = idx >> vb_log;
+                    *(float4*)(sm + tt * row_len + 3 * DIMP + (idx & (VB - 1))) = make_float4(pv[4 * i], pv[4 * i + 1], pv[4 * i + 2], pv[4 * i + 3]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < SCAN_PFK; ++i) {
+                const int idx = tid + i * nthr;
+                if (idx < nk) {
+                    const int tt = (idx >> dimp_log) / 3;
+                    sm[tt * row_len + (idx - tt * 3 * DIMP)] = pk[i];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < SCAN_PFV; ++i) {
+                const int idx = tid + i * nthr;
+                if (idx < nv) {
+                    const int tt = idx >> vb_log;
+                    sm[tt * row_len + 3 * DIMP + (idx & (VB - 1))] = pv[i];
+                }
             }
         }
         if (DELTA && tid < ct) sm[tid * row_len + 3 * DIMP + VB] = 1.0f / (1.0f + expf(-pb));
@@ -348,10 +402,10 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     while (lpc * R < dim) lpc <<= 1, ++lpc_log;
     const int cols = 64 / lpc, DIMP = lpc * R;
     const int waves_needed = (vdim + cols - 1) / cols;
-    // waves per workgroup: they share the staged k, q and decay.  Two, not more: a step is bound by instruction issue, and the
-    // launch's waves should spread over all SIMDs of the chip rather than stack up on the CUs of a few large workgroups
+    // waves per workgroup: they share the staged k, q and decay (fewer: the staging loads multiply; more: the launch's waves
+    // stack up on the CUs of a few large workgroups while a token's step is bound by instruction issue)
     int nw = 1;
-    while (nw < 2 && nw < waves_needed) nw <<= 1;
+    while (nw < 4 && nw < waves_needed) nw <<= 1;
     const int VB = nw * cols, nthr = nw * 64;
     int CT = SCAN_CT;                                            // tokens per staged chunk: what the prefetch registers and 48 KiB hold
     while (CT > 1 && ((CT * 3 * DIMP + nthr - 1) / nthr > SCAN_PFK || (CT * VB + nthr - 1) / nthr > SCAN_PFV ||
@@ -362,10 +416,19 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     const size_t lds = (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4;
     const dim3 grid(n_runs, heads, (vdim + VB - 1) / VB), block(nthr);
     QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
-#define QSV_SCAN(TQ, TB, DELTA)                                                                                              \
-    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA>), grid, block, lds, (hipStream_t)stream, o, (const TQ*)q, q_stride,  \
-                       (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state, runs, heads,  \
-                       qk_heads, dim, vdim, lpc_log, CT, q_scale)
+    const size_t el = qkv_dtype == QSV_F32 ? 4 : 2;
+    const bool vec = dim % 4 == 0 && vdim % 4 == 0 && VB % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 &&
+                     (uintptr_t)q % (4 * el) == 0 && (uintptr_t)k % (4 * el) == 0 && (uintptr_t)v % (4 * el) == 0 &&
+                     (uintptr_t)decay % 16 == 0;
+#define QSV_SCAN_V(TQ, TB, DELTA, VEC)                                                                                       \
+    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC>), grid, block, lds, (hipStream_t)stream, o, (const TQ*)q,      \
+                       q_stride, (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state,   \
+                       runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale)
+#define QSV_SCAN(TQ, TB, DELTA)                  \
+    do {                                         \
+        if (vec) QSV_SCAN_V(TQ, TB, DELTA, true); \
+        else QSV_SCAN_V(TQ, TB, DELTA, false);   \
+    } while (0)
     if (beta) {
         if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_SCAN(float, float, true);
         else if (qkv_dtype == QSV_F32 && beta_dtype == QSV_BF16) QSV_SCAN(float, bf16_t, true);
@@ -377,6 +440,7 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
         else QSV_REQUIRE(false, "qsv_recurrent_scan: operand type %d", qkv_dtype);
     }
 #undef QSV_SCAN
+#undef QSV_SCAN_V
     return qsv_launch_status("qsv_recurrent_scan");
 }
 
