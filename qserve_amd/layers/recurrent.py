@@ -1,7 +1,7 @@
 """Linear-recurrence mixers: a matrix state S [dim, vdim] per head and sequence, advanced token by token in float.
 
 GatedLinearAttention   S <- diag(a) S + k v^T;  o = S^T q          a = sigmoid(z)^(1 / tau) per key channel
-GatedDeltaRule         S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (the read-out sees the write)
+GatedDeltaRule         S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (o is read from the updated S)
                        g = exp(-exp(A_log) softplus(z + dt_bias)) per head and key channel, beta = sigmoid(.) per head,
                        q, k, v through a short causal convolution + silu, q and k made unit vectors per head
 

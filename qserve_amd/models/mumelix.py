@@ -11,7 +11,8 @@ layers: [{type, mixer: {...}, mlp: {kind: dense | moe, ...} | null}]}.
 * Mixers: `gla` (qserve_amd.layers.recurrent.GatedLinearAttention); `parallel` = attention with rotated keys and values
   (qserve_amd.layers.softmax_attention.RotatedValueAttention) beside a gated delta rule (GatedDeltaRule), joined by ParallelMixer.
 * Feed-forward: dense gated units or a top-k mixture of them (qserve_amd.layers.moe).
-* Layers loop.start .. loop.stop - 1 run loop.times times in a row with the same weights; every pass has its own cache and state.
+* `loop` repeats a block of consecutive layers: the layer order is [0, start) + [start, stop) x times + [stop, n).  A repeated
+  layer shares its weights between its runs, never its cache pools or states (`run_slices`).
 """
 import torch
 

@@ -270,7 +270,7 @@ MUMELIX = {
 
 def mumelix_config(s, m):
     mlp = {"kind": "moe", "expert": {"ff": s["ff"]}, "router": {"experts": s["experts"], "top": s["top"]}}
-    g = {"type": "gla", "mlp": mlp, "mixer": {"heads": m["g_heads"], "dim": m["g_dim"], "vdim": m["g_vdim"], "tau": 16.0}}
+    g = {"type": "gla", "mlp": mlp, "mixer": {"heads": m["g_heads"], "dim": m["g_dim"], "vdim": m["g_vdim"], "tau": 8.0}}
     rot = {"base": 500000.0, "dims": m["rot"], "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
     p = {"type": "parallel", "mlp": mlp,
          "mixer": {"left": {"heads": m["a_heads"], "kv_heads": m["a_kv"], "dim": m["a_dim"], "vdim": m["a_vdim"], "rot": rot,
