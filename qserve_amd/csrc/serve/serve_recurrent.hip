@@ -70,14 +70,13 @@ __global__ __launch_bounds__(NT) void conv_silu_unit_kernel(float* __restrict__ 
 
 // ---- the recurrence ---------------------------------------------------------------------------------------------------------
 // Columns of S (value channels) never meet: column j of head h needs k, q and the decay of the token and its own v_j.  A
-// workgroup owns a block of columns of one (run, head): a wave 64 / LPC of them, a lane R rows of one column; the LPC lanes of a
-// column are neighbours and add their partial dot products through DPP moves.  The run's tokens are walked in order, CT at
+// workgroup owns a block of columns of one (run, head): a wave 64 / LPC groups of NC of them, a lane R rows of its NC columns;
+// the LPC lanes of a column are neighbours and add their partial dot products through DPP moves.  The run's tokens are walked in order, CT at
 // a time: the workgroup stages k, q, the decay (float, zero-padded to LPC * R rows), its v columns and sigmoid(beta) of CT
 // tokens in LDS - the next CT tokens' values are already in registers while these are computed - so a token's step reads
 // LDS only, and the only exchange on the state's dependency chain is the delta rule's S^T k; the read-outs' partial sums wait
 // in registers until the chunk's end and are exchanged together.  The state is read once before and written once after (a run
 // that starts its sequence starts from zeros).
-constexpr int SCAN_R = 16;        // rows of a column per lane
 constexpr int SCAN_CT = 16;       // tokens per staged chunk, at most
 constexpr int SCAN_PFK = 24;      // staged k / q / decay values per thread and chunk, at most
 constexpr int SCAN_PFV = 16;      // staged v values per thread and chunk, at most
@@ -104,32 +103,34 @@ __device__ __forceinline__ float4 ld4(const bf16_t* p, size_t i) {
                        __uint_as_float(u.y & 0xffff0000u));
 }
 
-// VEC: dim, vdim, the row strides and the operands' addresses are multiples of four elements - staged four at a time
-template <typename TQ, typename TB, bool DELTA, bool VEC>
-__global__ __launch_bounds__(512) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
+// VEC: dim, vdim, the row strides and the operands' addresses are multiples of four elements - staged four at a time.
+// R rows and NC columns of the state per lane (with NC > 1 the token's k, q and decay rows are read from LDS once for NC columns).
+template <typename TQ, typename TB, bool DELTA, bool VEC, int R, int NC>
+__global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
                                                              const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
                                                              int64_t v_stride, const float* __restrict__ decay,
                                                              const TB* __restrict__ beta, int64_t beta_stride,
                                                              float* __restrict__ state, const int32_t* __restrict__ runs, int H,
                                                              int QH, int dim, int vdim, int lpc_log, int CT, float q_scale) {
-    constexpr int R = SCAN_R;
+    static_assert(R == 4 || R == 8 || R == 16, "rows per lane");
     extern __shared__ __attribute__((aligned(16))) float sm[];
     const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nthr >> 6;
-    const int lpc = 1 << lpc_log, cols = 64 >> lpc_log;
-    const int dimp_log = lpc_log + 4, DIMP = 1 << dimp_log, VB = nw * cols;       // (R = 16 = 2^4; nw and cols are powers of two)
+    const int lpc = 1 << lpc_log, cols = 64 >> lpc_log;                           // cols: column groups (of NC) per wave
+    const int dimp_log = lpc_log + (R == 16 ? 4 : R == 8 ? 3 : 2), DIMP = 1 << dimp_log, VB = nw * cols * NC;   // (all powers of two)
     const int vb_log = 31 - __clz(VB);
     const int row_len = 3 * DIMP + ((VB + 4) & ~3);              // floats of one staged token: k | q | decay | v | beta, 16-byte rows
-    const int part = lane & (lpc - 1), cb = wave * cols + (lane >> lpc_log);
-    const int j = blockIdx.z * VB + cb;
-    const bool col_ok = j < vdim;
+    const int part = lane & (lpc - 1), cb = (wave * cols + (lane >> lpc_log)) * NC;
+    const int j = blockIdx.z * VB + cb;                          // first of this lane's NC columns
     const int r0 = part * R;
     const int slot = runs[4 * blockIdx.x], first = runs[4 * blockIdx.x + 1], n = runs[4 * blockIdx.x + 2];
     const bool fresh = runs[4 * blockIdx.x + 3] == 0;
     const int h = blockIdx.y, qh = h / (H / QH);
-    float* Sg = state + (((size_t)slot * H + h) * dim) * (size_t)vdim + (col_ok ? j : 0);
-    float S[R];
+    float* Sg = state + (((size_t)slot * H + h) * dim) * (size_t)vdim;
+    float S[NC][R];
 #pragma unroll
-    for (int i = 0; i < R; ++i) S[i] = (!fresh && col_ok && r0 + i < dim) ? Sg[(size_t)(r0 + i) * vdim] : 0.f;
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int i = 0; i < R; ++i) S[c][i] = (!fresh && j + c < vdim && r0 + i < dim) ? Sg[(size_t)(r0 + i) * vdim + j + c] : 0.f;
 
     float pk[SCAN_PFK], pv[SCAN_PFV], pb = 0.f;
     // requests the operands of tokens [c0, c0 + ct) of the run into registers
@@ -235,13 +236,14 @@ __global__ __launch_bounds__(512) void recurrent_scan_kernel(float* __restrict__
         stage(ct);
         __syncthreads();
         if (c0 + CT < n) fetch(c0 + CT, min(CT, n - c0 - CT));   // in flight while this chunk is computed
-        float oacc[SCAN_CT];
+        float oacc[SCAN_CT][NC];
 #pragma unroll
         for (int tt = 0; tt < SCAN_CT; ++tt) {
-            oacc[tt] = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) oacc[tt][c] = 0.f;
             if (tt >= ct) continue;                              // (uniform)
             const float* row = sm + tt * row_len;
-            float kc[R], qc[R], gc[R];
+            float kc[R], qc[R], gc[R], vc[NC];
 #pragma unroll
             for (int i = 0; i < R; i += 4) {
                 const float4 a = *(const float4*)(row + r0 + i), b = *(const float4*)(row + DIMP + r0 + i),
@@ -250,41 +252,57 @@ __global__ __launch_bounds__(512) void recurrent_scan_kernel(float* __restrict__
                 qc[i] = b.x; qc[i + 1] = b.y; qc[i + 2] = b.z; qc[i + 3] = b.w;
                 gc[i] = c.x; gc[i + 1] = c.y; gc[i + 2] = c.z; gc[i + 3] = c.w;
             }
-            const float vc = row[3 * DIMP + cb];
-            float acc = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) vc[c] = row[3 * DIMP + cb + c];
             if (DELTA) {
+                const float bt = row[3 * DIMP + VB];
+                float acc[NC];
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    S[i] *= gc[i];
-                    acc += S[i] * kc[i];
+                for (int c = 0; c < NC; ++c) {
+                    acc[c] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < R; ++i) {
+                        S[c][i] *= gc[i];
+                        acc[c] += S[c][i] * kc[i];
+                    }
                 }
-                const float u = (vc - column_sum(acc, lpc)) * row[3 * DIMP + VB];
-                acc = 0.f;
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    S[i] += kc[i] * u;
-                    acc += S[i] * qc[i];
+                for (int c = 0; c < NC; ++c) {
+                    const float u = (vc[c] - column_sum(acc[c], lpc)) * bt;
+                    float a2 = 0.f;
+#pragma unroll
+                    for (int i = 0; i < R; ++i) {
+                        S[c][i] += kc[i] * u;
+                        a2 += S[c][i] * qc[i];
+                    }
+                    oacc[tt][c] = a2;
                 }
             } else {
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    S[i] = gc[i] * S[i] + kc[i] * vc;
-                    acc += S[i] * qc[i];
+                for (int c = 0; c < NC; ++c) {
+                    float a2 = 0.f;
+#pragma unroll
+                    for (int i = 0; i < R; ++i) {
+                        S[c][i] = gc[i] * S[c][i] + kc[i] * vc[c];
+                        a2 += S[c][i] * qc[i];
+                    }
+                    oacc[tt][c] = a2;
                 }
             }
-            oacc[tt] = acc;
         }
 #pragma unroll
-        for (int tt = 0; tt < SCAN_CT; ++tt) {
-            const float sum = column_sum(oacc[tt], lpc);
-            if (tt < ct && part == 0 && col_ok) o[((size_t)(first + c0 + tt) * H + h) * (size_t)vdim + j] = sum * q_scale;
-        }
+        for (int tt = 0; tt < SCAN_CT; ++tt)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const float sum = column_sum(oacc[tt][c], lpc);
+                if (tt < ct && part == 0 && j + c < vdim) o[((size_t)(first + c0 + tt) * H + h) * (size_t)vdim + j + c] = sum * q_scale;
+            }
     }
-    if (col_ok) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
 #pragma unroll
         for (int i = 0; i < R; ++i)
-            if (r0 + i < dim) Sg[(size_t)(r0 + i) * vdim] = S[i];
-    }
+            if (j + c < vdim && r0 + i < dim) Sg[(size_t)(r0 + i) * vdim + j + c] = S[c][i];
 }
 
 // ---- per-head RMS norm of the read-out, times a weight shared by the heads, times a gate ---------------------------------------
@@ -392,21 +410,29 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
                                   int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
                                   int beta_dtype, float* state, const int32_t* runs, int n_runs, int heads, int qk_heads, int dim,
                                   int vdim, float q_scale, void* stream) {
-    constexpr int R = SCAN_R;
     QSV_REQUIRE(o && q && k && v && decay && state && runs, "qsv_recurrent_scan: null argument");
-    QSV_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dim > 0 && dim <= 64 * R && vdim > 0 && n_runs >= 0 &&
+    // Rows of one column per lane: 8 while that leaves the launch at no more than ~2.5 waves per SIMD, else 16 (and for the tallest
+    // states).  Measured at 16 heads, 64 x 128 states: 8 x 1024 tokens (2048 / 1024 waves) 0.46 / 0.51 ms plain, 0.50 / 0.55 ms
+    // delta rule; 64 single tokens (16384 / 8192 waves) 56 / 43 us; two columns per lane 0.60 / 0.75 ms.  A token's step is a
+    // short chain of dependent instructions: up to the chip's fill, more and lighter waves win; beyond it, fewer and heavier ones.
+    int lpc8 = 1;
+    while (lpc8 * 8 < dim) lpc8 <<= 1;
+    const int64_t waves8 = (int64_t)n_runs * heads * (((int64_t)vdim * lpc8 + 63) / 64);
+    const int R = dim <= 64 * 8 && waves8 <= 2560 ? 8 : 16, NC = 1;
+    QSV_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dim > 0 && dim <= 64 * 16 && vdim > 0 && n_runs >= 0 &&
                     heads <= 65535,
                 "qsv_recurrent_scan: bad sizes (%d heads over %d, state %d x %d)", heads, qk_heads, dim, vdim);
     if (n_runs == 0) return QSV_OK;
     int lpc = 1, lpc_log = 0;
     while (lpc * R < dim) lpc <<= 1, ++lpc_log;
+    QSV_REQUIRE(lpc <= 64, "qsv_recurrent_scan: %d rows per lane for a state of %d rows", R, dim);
     const int cols = 64 / lpc, DIMP = lpc * R;
-    const int waves_needed = (vdim + cols - 1) / cols;
+    const int waves_needed = (vdim + cols * NC - 1) / (cols * NC);
     // waves per workgroup: they share the staged k, q and decay (fewer: the staging loads multiply; more: the launch's waves
     // stack up on the CUs of a few large workgroups while a token's step is bound by instruction issue)
     int nw = 1;
     while (nw < 4 && nw < waves_needed) nw <<= 1;
-    const int VB = nw * cols, nthr = nw * 64;
+    const int VB = nw * cols * NC, nthr = nw * 64;
     int CT = SCAN_CT;                                            // tokens per staged chunk: what the prefetch registers and 48 KiB hold
     while (CT > 1 && ((CT * 3 * DIMP + nthr - 1) / nthr > SCAN_PFK || (CT * VB + nthr - 1) / nthr > SCAN_PFV ||
                       (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4 > 48 * 1024))
@@ -420,14 +446,16 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     const bool vec = dim % 4 == 0 && vdim % 4 == 0 && VB % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 &&
                      (uintptr_t)q % (4 * el) == 0 && (uintptr_t)k % (4 * el) == 0 && (uintptr_t)v % (4 * el) == 0 &&
                      (uintptr_t)decay % 16 == 0;
-#define QSV_SCAN_V(TQ, TB, DELTA, VEC)                                                                                       \
-    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC>), grid, block, lds, (hipStream_t)stream, o, (const TQ*)q,      \
-                       q_stride, (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state,   \
-                       runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale)
-#define QSV_SCAN(TQ, TB, DELTA)                  \
-    do {                                         \
-        if (vec) QSV_SCAN_V(TQ, TB, DELTA, true); \
-        else QSV_SCAN_V(TQ, TB, DELTA, false);   \
+#define QSV_SCAN_V(TQ, TB, DELTA, VEC, RR, CC)                                                                               \
+    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC, RR, CC>), grid, block, lds, (hipStream_t)stream, o,            \
+                       (const TQ*)q, q_stride, (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta,         \
+                       beta_stride, state, runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale)
+#define QSV_SCAN(TQ, TB, DELTA)                                \
+    do {                                                       \
+        if (vec && R == 8) QSV_SCAN_V(TQ, TB, DELTA, true, 8, 1);   \
+        else if (R == 8) QSV_SCAN_V(TQ, TB, DELTA, false, 8, 1);    \
+        else if (vec) QSV_SCAN_V(TQ, TB, DELTA, true, 16, 1);       \
+        else QSV_SCAN_V(TQ, TB, DELTA, false, 16, 1);               \
     } while (0)
     if (beta) {
         if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_SCAN(float, float, true);
