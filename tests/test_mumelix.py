@@ -610,3 +610,29 @@ def test_gated_expert_forms_agree_in_bfloat16(E, top, ff, D, T):
             setattr(o, k, v)
         y = o.moe_experts(h.to(dev), w_in, down.to(dev), idx.to(dev), wt.to(dev), act="swiglu").double().cpu()
         assert_close(y, ref, 2e-2, f"{name} form")
+
+
+# ---- host logic alone ------------------------------------------------------------------------------------------------------------
+
+def test_state_rows_swap_per_step_and_follow_the_slot():
+    from qserve_amd.serving.cache import PagedCache, StateSpec
+    cache = PagedCache([4, (3, 6)], num_pages=4, max_seqs=3, dtype=torch.float32, device="cpu", page=64,
+                       states=[StateSpec((2, 5)), StateSpec((7,), copies=2)])
+    assert cache.pools[0].shape == (256, 4) and cache.pools[1].shape == (3, 256, 6)
+    assert cache.states[0].shape == (3, 2, 5) and cache.states[1].shape == (6, 7)
+    a, b = cache.admit(), cache.admit()
+    r1, w1 = cache.step_rows(b)
+    r2, w2 = cache.step_rows(b)
+    assert {r1, w1} == {2 * b, 2 * b + 1} and (r2, w2) == (w1, r1)          # the next step reads what this one wrote
+    assert set(cache.step_rows(a)) == {2 * a, 2 * a + 1}
+    cfg = make_config([gla()], width=8, vocab=11)
+    eng = build_engine(cfg, f32(P.random_weights(cfg)), "unfused", max_tokens=128, max_seqs=2)
+    s0, s1 = eng.open_sequence(), eng.open_sequence()
+    batch = eng.layout([(s1, [1, 2, 3]), (s0, [4])])
+    assert batch.run_off.tolist() == [0, 1, 2, 0] and batch.state_rd.tolist() == [-1] * 4          # both sequences start here
+    assert batch.state_wr.tolist()[:2] == [-1, -1] and batch.state_wr.tolist()[2] in (2 * s1, 2 * s1 + 1)
+    assert batch.runs().tolist() == [[s1, 0, 3, 0], [s0, 3, 1, 0]]
+    nxt = eng.layout([(s1, [5, 6])])
+    assert nxt.state_rd.tolist() == [batch.state_wr.tolist()[2]] * 2 and nxt.runs().tolist() == [[s1, 0, 2, 3]]
+    with pytest.raises(ValueError):
+        eng.layout([(s0, [1]), (s0, [2])])
