@@ -49,15 +49,17 @@ int qsv_latent_query(float* qf, const void* q, const void* q_abs, const float* r
 /* Softmax attention of every token over the cached latent rows of its sequence:
  *   score(t, h, j) = qf[t, h] . pool[row(seq[t], j)]   for  max(0, pos[t] - window + 1) <= j <= pos[t]  (window 0: all j <= pos)
  *   out[t, h]      = sum_j softmax_j(score) * pool[row][0 : rank]            (storage type, [T, H, rank])
- * row(s, j) = block_table[s * table_stride + j / page] * page + j % page.  variant: 0 = default kernel choice. */
+ * row(s, j) = block_table[s * table_stride + j / page] * page + j % page.  variant: 0 = default kernel choice.
+ * Several pools in one launch: heads [g * heads_per_pool, (g + 1) * heads_per_pool) read the pool that starts pool_stride
+ * elements after pool g - 1 (one pool for all heads: heads_per_pool = heads, pool_stride = 0). */
 int qsv_latent_attention(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                          const int32_t* seq, const int32_t* pos, int window, int n_tokens, int heads, int rank,
-                         int row_width, int page, int dtype, int variant, void* stream);
+                         int row_width, int page, int heads_per_pool, int64_t pool_stride, int dtype, int variant, void* stream);
 
 int qsv_latent_attention_tile_tokens(int heads);
 int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
 /* The same attention on the bf16 matrix cores.  The host cuts every sequence's tokens of the step into work tiles of at most
- * qsv_latent_attention_tile_tokens(heads) consecutive tokens: tiles int32 [n_tiles, 3] = (sequence slot, first flat token
+ * qsv_latent_attention_tile_tokens(heads_per_pool) consecutive tokens: tiles int32 [n_tiles, 3] = (sequence slot, first flat token
  * index, tokens).  qsv_latent_attention_mfma_ok() says whether the sizes are taken (bfloat16 storage, rank and row width
  * multiples of 8, row width <= 576); otherwise use qsv_latent_attention. * key_splits > 1 cuts every tile's keys over that many workgroups and merges the partial results in a second launch (steps
  * with few tiles: decoding); part_o (float [key_splits, n_tokens, heads, rank]) and part_ml (float [key_splits, n_tokens,
@@ -66,7 +68,7 @@ int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
 int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                               const int32_t* pos, const int32_t* tiles, int n_tiles, int window, int heads, int rank,
                               int row_width, int page, int key_splits, float* part_o, float* part_ml, int n_tokens,
-                              int q_first, void* stream);
+                              int q_first, int heads_per_pool, int64_t pool_stride, void* stream);
 
 /* o[t, i] *= sigmoid(g[t * g_stride + i]),  i < n. */
 int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int n, int dtype, void* stream);

@@ -28,10 +28,10 @@ __device__ __forceinline__ unsigned pack_bf2(float a, float b) { return (unsigne
 // RT: 32-element steps along a cache row (R <= 32 RT); CT: 16-column tiles of the output (rank <= 16 CT).
 template <int RT, int CT>
 __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_mfma_kernel(
-    bf16_t* __restrict__ out, const float* __restrict__ qf, const bf16_t* __restrict__ pool,
+    bf16_t* __restrict__ out, const float* __restrict__ qf, const bf16_t* __restrict__ pool_base,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ pos, const int32_t* __restrict__ tiles,
     int window, int H, int rank, int R, int page, int HP, int TQ, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int n_tokens, int s_lo, int s_hi) {
+    int n_tokens, int s_lo, int s_hi, int per, int64_t pool_stride) {
     constexpr int RS = 32 * RT + 8;                      // row stride (elements) of the row-major tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* Ks = (bf16_t*)smem;                          // [BN][RS]
@@ -41,7 +41,10 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int col = lane & 15, g4 = lane >> 4;           // query row of this lane; k-group / accumulator row block
     const int slot = tiles[3 * blockIdx.x], t0 = tiles[3 * blockIdx.x + 1], ntok = tiles[3 * blockIdx.x + 2];
-    const int h0 = blockIdx.y * 16;
+    // heads [g per, (g + 1) per) read pool g (pool_stride elements apart): blockIdx.y walks the pools' head groups of 16
+    const int gpp = (per + 15) / 16, pool_id = blockIdx.y / gpp;
+    const int h0 = pool_id * per + (blockIdx.y % gpp) * 16, h_end = pool_id * per + per;
+    const bf16_t* __restrict__ pool = pool_base + (size_t)pool_id * (size_t)pool_stride;
     const int32_t* bt = block_table + (size_t)slot * table_stride;
 
     // rows of this wave: group grp of TQ tokens, key split sp
@@ -51,7 +54,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     const int grp = active ? w % G : 0, sp = active ? w / G : 0;
     const int tok_in = grp * TQ + col / HP;              // token of this lane's query row within the tile
     const int head = h0 + col % HP;
-    const bool row_ok = active && tok_in < ntok && head < H;
+    const bool row_ok = active && tok_in < ntok && head < h_end;
     const int t = t0 + (tok_in < ntok ? tok_in : 0);
     const int p_row = pos[t];
     const int lo_row = window > 0 ? max(0, p_row - window + 1) : 0;
@@ -301,15 +304,17 @@ extern "C" int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype) 
 extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table,
                                          int table_stride, const int32_t* pos, const int32_t* tiles, int n_tiles, int window,
                                          int H, int rank, int R, int page, int key_splits, float* part_o, float* part_ml,
-                                         int n_tokens, int q_first, void* stream) {
+                                         int n_tokens, int q_first, int heads_per_pool, int64_t pool_stride, void* stream) {
     QSV_REQUIRE(out && qf && pool && block_table && pos && tiles, "qsv_latent_attention_mfma: null argument");
     QSV_REQUIRE(qsv_latent_attention_mfma_ok(rank, R, QSV_BF16) && R >= rank && H > 0 && page > 0 && page % BN == 0 && window >= 0 && n_tiles >= 0,
                 "qsv_latent_attention_mfma: sizes not supported (rank %d, row %d)", rank, R);
     if (n_tiles == 0) return QSV_OK;
-    const Geometry g = geometry(H);
+    QSV_REQUIRE(heads_per_pool > 0 && H % heads_per_pool == 0 && pool_stride >= 0,
+                "qsv_latent_attention_mfma: %d heads over pools of %d", H, heads_per_pool);
+    const Geometry g = geometry(heads_per_pool);
     QSV_REQUIRE(key_splits >= 1 && key_splits <= 64 && (key_splits == 1 || (part_o && part_ml && n_tokens > 0)),
                 "qsv_latent_attention_mfma: key splits without workspace");
-    const dim3 grid(n_tiles, (H + 15) / 16, key_splits), block(64 * NWV);
+    const dim3 grid(n_tiles, (H / heads_per_pool) * ((heads_per_pool + 15) / 16), key_splits), block(64 * NWV);
     QSV_REQUIRE(q_first >= 0 && q_first < R, "qsv_latent_attention_mfma: first query element %d of %d", q_first, R);
     const int rt = (R + 31) / 32, ct = (rank + 15) / 16;
     const int s_lo = q_first / 32, s_hi = rt;
@@ -325,7 +330,7 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
         }                                                                                                                    \
         hipLaunchKernelGGL((latent_attention_mfma_kernel<RT, CT>), grid, block, lds, (hipStream_t)stream, (bf16_t*)out, qf,  \
                            (const bf16_t*)pool, block_table, table_stride, pos, tiles, window, H, rank, R, page, g.HP, g.TQ, \
-                           part_o, part_ml, n_tokens, s_lo, s_hi);                                                           \
+                           part_o, part_ml, n_tokens, s_lo, s_hi, heads_per_pool, pool_stride);                              \
     } while (0)
     if (rt <= 4 && ct <= 8) QSV_MFMA(4, 8);
     else if (rt <= 6 && ct <= 12) QSV_MFMA(6, 12);

@@ -96,16 +96,19 @@ class HipOps:
     def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0):
         """batch: the step's StepBatch (block table, sequence slot and position per token, work tiles).  variant: 0 = the
         matrix-core kernel where it takes the sizes, 1 = always the wave kernel.  key_splits: None = chosen from the number
-        of workgroups and the context.  q_first: the caller's promise that every query is zero before that element."""
+        of workgroups and the context.  q_first: the caller's promise that every query is zero before that element.
+        pool [rows, R]: one pool for all heads; [G, rows, R]: head h reads pool h // (H / G), all in one launch."""
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         self._need(qf, pool, block_table, seq, pos)
         assert pool.size(-1) == R and block_table.dtype == torch.int32 and seq.dtype == torch.int32
+        per, pool_stride = (H, 0) if pool.dim() == 2 else (H // pool.size(0), pool.stride(0))
+        assert pool.dim() == 2 or H % pool.size(0) == 0
         if variant == 0 and page % 32 == 0 and self.L.qsv_latent_attention_mfma_ok(rank, R, self.code):
-            tiles = batch.tiles(self.L.qsv_latent_attention_tile_tokens(H))
+            tiles = batch.tiles(self.L.qsv_latent_attention_tile_tokens(per))
             # few workgroups and long contexts (decoding): cut the keys over several workgroups, merged by a second launch
-            groups = tiles.size(0) * ((H + 31) // 32)
+            groups = tiles.size(0) * (H // per) * ((per + 31) // 32)
             span = min(batch.max_pos + 1, int(window)) if window else batch.max_pos + 1
             # (rows wider than 320 elements: one workgroup per CU at a time - a launch of one round of workgroups is the aim)
             target = self.attention_split_target // 2 if R > 320 else self.attention_split_target
@@ -118,11 +121,11 @@ class HipOps:
                                                         block_table.stride(0), pos.data_ptr(), tiles.data_ptr(), tiles.size(0),
                                                         int(window or 0), H, rank, R, page, splits,
                                                         0 if po is None else po.data_ptr(), 0 if pm is None else pm.data_ptr(), T,
-                                                        int(q_first), self._s()), "latent_attention_mfma")
+                                                        int(q_first), per, pool_stride, self._s()), "latent_attention_mfma")
             return out
         self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
-                                               rank, R, page, self.code, variant, self._s()), "latent_attention")
+                                               rank, R, page, per, pool_stride, self.code, variant, self._s()), "latent_attention")
         return out
 
     def sigmoid_gate(self, o, g):
@@ -460,13 +463,17 @@ class TorchOps:
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         bt = block_table.long()
+        pools = [pool] if pool.dim() == 2 else list(pool)
+        per = H // len(pools)
         for t in range(T):
             p = int(pos[t])
             lo = max(0, p - window + 1) if window else 0
             j = torch.arange(lo, p + 1, device=qf.device)
-            rows = pool[bt[int(seq[t]), j // page] * page + j % page].float()        # [n, R]
-            w = torch.softmax(qf[t] @ rows.t(), dim=-1)                              # [H, n]
-            out[t] = (w @ rows[:, :rank]).to(self.dtype)
+            at = bt[int(seq[t]), j // page] * page + j % page
+            for g, pl in enumerate(pools):
+                rows = pl[at].float()                                                # [n, R]
+                w = torch.softmax(qf[t, g * per:(g + 1) * per] @ rows.t(), dim=-1)   # [per, n]
+                out[t, g * per:(g + 1) * per] = (w @ rows[:, :rank]).to(self.dtype)
         return out
 
     def sigmoid_gate(self, o, g):

@@ -7,7 +7,7 @@ dimensions of every q and k head turn with the position (halves layout, table `r
 
 Cache: per key / value head one pool of rows [v (vdim) | k (dim)].  The attention itself is the paged row-attention kernel of
 the latent layers (qserve_amd.layers.latent_attention): a query [0 (vdim) | q * scale] against such rows scores q . k, and
-the softmax-weighted sum of the rows' first vdim elements is the output.
+the softmax-weighted sum of the rows' first vdim elements is the output; one launch serves all key / value heads.
 """
 import torch
 
@@ -36,13 +36,6 @@ class RotatedValueAttention:
         proj = linear(h, self.w_in)
         qf = ops.attention_prep(proj, 0, H * self.dim, (H + G) * self.dim, H, G, self.dim, self.vdim, self.rot_n,
                                 self.rope_k.reserve(n), self.rope_v.reserve(n), self.scale, pool, batch)
-        per = H // G
-        if G == 1:
-            o = ops.latent_attention(qf, pool[0], batch, None, self.vdim, self.page, q_first=self.vdim)
-        else:
-            o = torch.empty((T, H, self.vdim), dtype=h.dtype, device=h.device)
-            for g in range(G):
-                o[:, g * per:(g + 1) * per] = ops.latent_attention(qf[:, g * per:(g + 1) * per].contiguous(), pool[g], batch, None,
-                                                                   self.vdim, self.page, q_first=self.vdim)
+        o = ops.latent_attention(qf, pool, batch, None, self.vdim, self.page, q_first=self.vdim)      # head h reads pool h // (H / G)
         ops.rotate_heads(o, self.rope_v.table, batch.pos, -1.0)
         return linear(o.view(T, H * self.vdim), self.w_o)

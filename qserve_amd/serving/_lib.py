@@ -17,10 +17,10 @@ SIGNATURES = {
     "qsv_layer_norm_rows": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _vp]),
     "qsv_latent_prep": (_i, [_vp, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _i, _vp]),
     "qsv_latent_query": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "qsv_latent_attention": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "qsv_latent_attention": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _i, _vp]),
     "qsv_latent_attention_tile_tokens": (_i, [_i]),
     "qsv_latent_attention_mfma_ok": (_i, [_i, _i, _i]),
-    "qsv_latent_attention_mfma": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
+    "qsv_latent_attention_mfma": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _i, _i64, _vp]),
     "qsv_sigmoid_gate": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp]),
     "qsv_moe_route": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "qsv_moe_up": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),

@@ -95,7 +95,7 @@ def test_serve_argument_validation_without_gpu():
     L = lib()
     assert L.qsv_moe_route(1, 1, 1, 1, None, 0, 4, 64, 8, 3, 4, 1, 0, None) == 1  # top 3 of one kept group of 2
     assert b"experts" in L.qsv_last_error()
-    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 1000, 1032, 64, 0, 1, None) == 1   # rows wider than 1024
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 1000, 1032, 64, 2, 0, 0, 1, None) == 1   # rows wider than 1024
     assert L.qsv_latent_attention_mfma_ok(64, 80, 0) == 1 and L.qsv_latent_attention_mfma_ok(64, 80, 1) == 0
     assert L.qsv_latent_attention_mfma_ok(70, 70, 0) == 0
     assert [L.qsv_latent_attention_tile_tokens(h) for h in (1, 3, 6, 16, 32, 40)] == [64, 16, 8, 4, 4, 4]

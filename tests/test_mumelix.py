@@ -159,6 +159,7 @@ def test_gated_linear_attention_alone(backend):
     _mixer_alone(backend, gla(), 40, [1, 3, 17, 18, 39])
     _mixer_alone(backend, gla(heads=1, dim=40, vdim=70, tau=1.0), 21, [2, 4])         # a column split over several lanes, two column blocks
     _mixer_alone(backend, gla(heads=5, dim=3, vdim=2, tau=30.0), 9, [8])
+    _mixer_alone(backend, gla(), 120, [15, 31, 48, 81])             # runs of 15, 16, 17, 33, 39 tokens: the kernel stages 16 at a time
 
 
 def test_parallel_mixer_alone(backend):
@@ -167,6 +168,7 @@ def test_parallel_mixer_alone(backend):
     _mixer_alone(backend, par(taps=1, r_kv=1, kv_heads=4, rot_dims=12), 14, [5])     # no history; one q/k head for all; every dimension turns
     _mixer_alone(backend, par(taps=6, r_heads=3, r_kv=3, r_dim=20, r_vdim=3, heads=1, kv_heads=1, dim=4, vdim=2, rot_dims=2), 30, [3, 4, 6, 13])
     _mixer_alone(backend, par(), 150, [63, 64, 65, 129])                              # page borders
+    _mixer_alone(backend, par(r_dim=40, r_vdim=70), 120, [15, 31, 48, 81])            # staging chunk edges; columns over two blocks
 
 
 def test_stream_norm_and_token_shift(backend):
