@@ -106,11 +106,11 @@ int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, c
                     int n_experts, int rows, int K, int act, void* stream);
 /* Grouped expert product on the bf16 matrix cores (prompt phase): the same out[s, n] for work tiles (expert, first sorted slot,
  * slots <= qsv_grouped_gemm_tile_slots()) listed in tiles int32 [n_tiles, 3]; K a multiple of qsv_grouped_gemm_k_step(), n_rows
- * a multiple of 4, n_tiles <= 65535. */
+ * a multiple of 4, n_tiles <= 65535.  act: QSV_ACT_* (QSV_ACT_GLU: out is n_rows / 2 wide). */
 int qsv_grouped_gemm_tile_slots(void);
 int qsv_grouped_gemm_k_step(void);
 int qsv_grouped_gemm(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int32_t* tiles,
-                     int n_tiles, int n_rows, int K, int relu_sq, void* stream);
+                     int n_tiles, int n_rows, int K, int act, void* stream);
 int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, int n_rows, int width, int dtype, void* stream);
 int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream);
 int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n_tokens, int top_k, int width,

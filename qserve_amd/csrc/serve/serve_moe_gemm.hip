@@ -5,7 +5,7 @@
 // both operands are contiguous along the reduction, so with the weight rows as the A operand and the slots' inputs as the B
 // operand (v_mfma_f32_16x16x32_bf16) a lane ends up with 4 consecutive n of one slot - an 8-byte store.  The input row of a
 // slot is fetched through an index (the gather into sorted order is part of the load), relu(.)^2 is the epilogue of the first
-// product.  K steps of 64 through LDS (stride 72 elements: conflict-free 16-byte reads), the next step's pieces in flight in
+// product (or the gated unit: gate and up rows interleaved in the weight).  K steps of 64 through LDS (stride 72 elements: conflict-free 16-byte reads), the next step's pieces in flight in
 // registers while this one is multiplied.
 #include "serve_common.h"
 
@@ -25,7 +25,9 @@ constexpr int NPA = BNW * CPR / 256, NPB = BS * CPR / 256;   // pieces per threa
 
 __device__ __forceinline__ unsigned pack_bf2(float a, float b) { return (unsigned)f2bf(a) | ((unsigned)f2bf(b) << 16); }
 
-template <bool RELU_SQ>
+// ACT: 0 nothing, 1 relu^2, 2 gated unit - weight rows 2f (gate) and 2f + 1 (up) are neighbours, so a lane's four rows are two
+// whole units: out[s, f] = silu(gate) * up, N / 2 wide
+template <int ACT>
 __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
                                                            const int64_t* __restrict__ x_index, int div,
                                                            const bf16_t* __restrict__ W, const int32_t* __restrict__ tiles, int N,
@@ -108,7 +110,12 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict
             const int n = n0 + 16 * MT * w + 16 * mt + 4 * g4;
             if (n >= N) continue;                                   // N % 4 == 0: the four rows are inside together
             v4f v = acc[mt][nt];
-            if (RELU_SQ) {
+            if (ACT == 2) {
+                const float u0 = v[0] / (1.0f + expf(-v[0])) * v[1], u1 = v[2] / (1.0f + expf(-v[2])) * v[3];
+                *(unsigned*)(out + (size_t)(s_first + sl) * (N / 2) + n / 2) = pack_bf2(u0, u1);
+                continue;
+            }
+            if (ACT == 1) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const float x = fmaxf(v[r], 0.f);
@@ -127,17 +134,19 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict
 extern "C" int qsv_grouped_gemm_tile_slots(void) { return BS; }
 extern "C" int qsv_grouped_gemm_k_step(void) { return KS; }
 extern "C" int qsv_grouped_gemm(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int32_t* tiles,
-                                int n_tiles, int N, int K, int relu_sq, void* stream) {
+                                int n_tiles, int N, int K, int act, void* stream) {
     QSV_REQUIRE(out && X && W && tiles && div > 0 && n_tiles >= 0, "qsv_grouped_gemm: bad arguments");
     QSV_REQUIRE(N > 0 && N % 4 == 0 && K > 0 && K % KS == 0, "qsv_grouped_gemm: N %d (a multiple of 4), K %d (a multiple of 64)", N, K);
     QSV_REQUIRE(n_tiles <= 65535, "qsv_grouped_gemm: %d tiles (at most 65535 per launch)", n_tiles);
+    QSV_REQUIRE(act == QSV_ACT_NONE || act == QSV_ACT_RELU_SQ || act == QSV_ACT_GLU, "qsv_grouped_gemm: activation %d", act);
     if (n_tiles == 0) return QSV_OK;
     const dim3 grid((N + BNW - 1) / BNW, n_tiles), block(256);
-    if (relu_sq)
-        hipLaunchKernelGGL(grouped_gemm_kernel<true>, grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, x_index,
-                           div, (const bf16_t*)W, tiles, N, K);
-    else
-        hipLaunchKernelGGL(grouped_gemm_kernel<false>, grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, x_index,
-                           div, (const bf16_t*)W, tiles, N, K);
+#define QSV_GG(ACT)                                                                                                          \
+    hipLaunchKernelGGL(grouped_gemm_kernel<ACT>, grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, x_index, div, \
+                       (const bf16_t*)W, tiles, N, K)
+    if (act == QSV_ACT_RELU_SQ) QSV_GG(1);
+    else if (act == QSV_ACT_GLU) QSV_GG(2);
+    else QSV_GG(0);
+#undef QSV_GG
     return qsv_launch_status("qsv_grouped_gemm");
 }

@@ -343,7 +343,8 @@ class HipOps:
         return y
 
     def _moe_experts_sorted(self, h, up, down, idx, wt, code=1):
-        """code = 2 (gated units): the first product leaves both halves of every unit ([n, 2 ff]), `glu` folds them."""
+        """code = 2 (gated units): the grouped kernel folds the two halves of a unit in its epilogue; with vendor products the
+        first product leaves both halves ([n, 2 ff]) and `glu` folds them."""
         T, D = h.shape
         E, rows, K = up.size(0), up.size(1), idx.size(1)
         ff = rows // 2 if code == 2 else rows
@@ -360,15 +361,12 @@ class HipOps:
             for e, c in enumerate(counts):
                 tiles += [(e, a + o, min(ts, c - o)) for o in range(0, c, ts)]
                 a += c
-            act = torch.empty((n, rows), dtype=self.dtype, device=h.device)
+            act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
             ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
-            tls = [torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device) for lo in range(0, len(tiles), 65535)]
-            for tl in tls:
+            for lo in range(0, len(tiles), 65535):
+                tl = torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device)
                 self.check(self.L.qsv_grouped_gemm(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), tl.data_ptr(),
-                                                   tl.size(0), rows, D, 1 if code == 1 else 0, self._s()), "grouped_gemm(up)")
-            if code == 2:
-                act = self.glu(act)
-            for tl in tls:
+                                                   tl.size(0), rows, D, code, self._s()), "grouped_gemm(up)")
                 self.check(self.L.qsv_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), tl.data_ptr(),
                                                    tl.size(0), D, ff, 0, self._s()), "grouped_gemm(down)")
             y = torch.empty((T, D), dtype=self.dtype, device=h.device)
