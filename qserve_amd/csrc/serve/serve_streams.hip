@@ -79,6 +79,108 @@ __global__ __launch_bounds__(NT) void hc_write_kernel(float* __restrict__ x, con
     }
 }
 
+// ---- the same two kernels for widths that are multiples of four: 16-byte stream accesses, four elements per thread and pass ----
+__device__ __forceinline__ void ld4t(const float* p, size_t i, float (&v)[4]) {
+    const float4 a = *(const float4*)(p + i);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void ld4t(const bf16_t* p, size_t i, float (&v)[4]) {
+    const uint2 u = *(const uint2*)(p + i);
+    v[0] = __uint_as_float(u.x << 16); v[1] = __uint_as_float(u.x & 0xffff0000u);
+    v[2] = __uint_as_float(u.y << 16); v[3] = __uint_as_float(u.y & 0xffff0000u);
+}
+__device__ __forceinline__ void st4t(float* p, size_t i, const float (&v)[4]) { *(float4*)(p + i) = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void st4t(bf16_t* p, size_t i, const float (&v)[4]) {
+    *(uint2*)(p + i) = make_uint2((unsigned)f2bf(v[0]) | ((unsigned)f2bf(v[1]) << 16), (unsigned)f2bf(v[2]) | ((unsigned)f2bf(v[3]) << 16));
+}
+__device__ __forceinline__ void stream_sum4(const float* __restrict__ x, const float* __restrict__ w_in, size_t t, int S, int D, int i,
+                                            float (&u)[4]) {
+    u[0] = u[1] = u[2] = u[3] = 0.f;
+    for (int s = 0; s < S; ++s) {
+        float v[4];
+        ld4t(x, (t * S + s) * D + i, v);
+        const float w = w_in[s];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) u[j] += w * v[j];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void hc_read_vec_kernel(T* __restrict__ h, const float* __restrict__ x, const float* __restrict__ w_in,
+                                                         const T* __restrict__ nw, const T* __restrict__ nb, float alpha,
+                                                         const T* __restrict__ shift, float* __restrict__ prev,
+                                                         const int32_t* __restrict__ run_off, const int32_t* __restrict__ state_rd,
+                                                         const int32_t* __restrict__ state_wr, int S, int D) {
+    const size_t t = blockIdx.x;
+    const bool shifted = shift != nullptr;
+    const int off = shifted ? run_off[t] : 0, rd = shifted ? state_rd[t] : -1, wr = shifted ? state_wr[t] : -1;
+    for (int i = threadIdx.x * 4; i < D; i += NT * 4) {
+        float w[4], b[4], u[4], n[4];
+        ld4t(nw, i, w);
+        ld4t(nb, i, b);
+        stream_sum4(x, w_in, t, S, D, i, u);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) n[j] = tanhf(alpha * u[j]) * w[j] + b[j];
+        if (shifted) {
+            float before[4] = {0.f, 0.f, 0.f, 0.f}, mu[4];
+            if (off > 0) {
+                stream_sum4(x, w_in, t - 1, S, D, i, u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) before[j] = tanhf(alpha * u[j]) * w[j] + b[j];
+            } else if (rd >= 0) {
+                ld4t(prev, (size_t)rd * D + i, before);
+            }
+            if (wr >= 0) st4t(prev, (size_t)wr * D + i, n);
+            ld4t(shift, i, mu);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) n[j] += (before[j] - n[j]) * mu[j];
+        }
+        st4t(h, t * D + i, n);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void hc_write_vec_kernel(float* __restrict__ x, const T* __restrict__ y, const float* __restrict__ mix,
+                                                          const float* __restrict__ w_out, int S, int D, T* __restrict__ h_next,
+                                                          const float* __restrict__ w_in_next, const T* __restrict__ nw,
+                                                          const T* __restrict__ nb, float alpha) {
+    const size_t t = blockIdx.x;
+    for (int i = threadIdx.x * 4; i < D; i += NT * 4) {
+        float old[MAX_STREAMS][4], yv[4], u[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < MAX_STREAMS; ++s)
+            if (s < S) ld4t(x, (t * S + s) * D + i, old[s]);
+        ld4t(y, t * D + i, yv);
+        for (int r = 0; r < S; ++r) {
+            float a[4];
+            const float wo = w_out[r];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) a[j] = wo * yv[j];
+#pragma unroll
+            for (int s = 0; s < MAX_STREAMS; ++s)
+                if (s < S) {
+                    const float m = mix[s * S + r];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) a[j] += m * old[s][j];
+                }
+            st4t(x, (t * S + r) * D + i, a);
+            if (h_next) {
+                const float wi = w_in_next[r];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u[j] += wi * a[j];
+            }
+        }
+        if (h_next) {
+            float w[4], b[4], n[4];
+            ld4t(nw, i, w);
+            ld4t(nb, i, b);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) n[j] = tanhf(alpha * u[j]) * w[j] + b[j];
+            st4t(h_next, t * D + i, n);
+        }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void dyt_sum_rows_kernel(T* __restrict__ out, const float* __restrict__ x,
                                                           const int32_t* __restrict__ rows, const T* __restrict__ nw,
@@ -137,9 +239,15 @@ extern "C" int qsv_hc_read(void* h, const float* x, const float* w_in, const voi
     QSV_REQUIRE(h && x && w_in && norm_w && norm_b && n >= 0 && D > 0 && streams > 0, "qsv_hc_read: bad arguments");
     QSV_REQUIRE(!shift || (prev && run_off && state_rd && state_wr), "qsv_hc_read: token shift without its state");
     if (n == 0) return QSV_OK;
-    QSV_DISPATCH(dtype, "qsv_hc_read",
-                 hipLaunchKernelGGL(hc_read_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, (T*)h, x, w_in, (const T*)norm_w,
-                                    (const T*)norm_b, alpha, (const T*)shift, prev, run_off, state_rd, state_wr, streams, D));
+    if (D % 4 == 0)
+        QSV_DISPATCH(dtype, "qsv_hc_read",
+                     hipLaunchKernelGGL(hc_read_vec_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, (T*)h, x, w_in,
+                                        (const T*)norm_w, (const T*)norm_b, alpha, (const T*)shift, prev, run_off, state_rd, state_wr,
+                                        streams, D));
+    else
+        QSV_DISPATCH(dtype, "qsv_hc_read",
+                     hipLaunchKernelGGL(hc_read_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, (T*)h, x, w_in, (const T*)norm_w,
+                                        (const T*)norm_b, alpha, (const T*)shift, prev, run_off, state_rd, state_wr, streams, D));
     return qsv_launch_status("qsv_hc_read");
 }
 
@@ -149,9 +257,14 @@ extern "C" int qsv_hc_write(float* x, const void* y, const float* mix, const flo
     QSV_REQUIRE(!h_next || (w_in_next && norm_w && norm_b), "qsv_hc_write: the next sublayer's input without its weights");
     QSV_REQUIRE(streams > 0 && streams <= MAX_STREAMS, "qsv_hc_write: %d streams (at most %d)", streams, MAX_STREAMS);
     if (n == 0) return QSV_OK;
-    QSV_DISPATCH(dtype, "qsv_hc_write",
-                 hipLaunchKernelGGL(hc_write_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (const T*)y, mix, w_out,
-                                    streams, D, (T*)h_next, w_in_next, (const T*)norm_w, (const T*)norm_b, alpha));
+    if (D % 4 == 0)
+        QSV_DISPATCH(dtype, "qsv_hc_write",
+                     hipLaunchKernelGGL(hc_write_vec_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (const T*)y, mix, w_out,
+                                        streams, D, (T*)h_next, w_in_next, (const T*)norm_w, (const T*)norm_b, alpha));
+    else
+        QSV_DISPATCH(dtype, "qsv_hc_write",
+                     hipLaunchKernelGGL(hc_write_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (const T*)y, mix, w_out,
+                                        streams, D, (T*)h_next, w_in_next, (const T*)norm_w, (const T*)norm_b, alpha));
     return qsv_launch_status("qsv_hc_write");
 }
 
