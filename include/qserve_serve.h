@@ -157,11 +157,12 @@ int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, in
  *   beta == NULL:  S <- diag(g) S + k v^T                                  o = S^T q * q_scale
  *   else:          S <- diag(g) S;  u = sigmoid(beta[t, head]) (v - S^T k);  S <- S + k u^T;  o = S^T q * q_scale
  * q, k: [T, qk_heads, dim] (head h reads h / (heads / qk_heads)), v: [T, heads, vdim], each with its row stride, of type
- * qkv_dtype; o: float [T, heads, vdim]. */
+ * qkv_dtype; o: float [T, heads, vdim].  max_run: the longest run's tokens as the host knows them (1: every run is one decoded
+ * token - a kernel without staging is used; any larger value, or 0 for unknown: the general kernel). */
 int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                        int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
-                       int beta_dtype, float* state, const int32_t* runs, int n_runs, int heads, int qk_heads, int dim,
-                       int vdim, float q_scale, void* stream);
+                       int beta_dtype, float* state, const int32_t* runs, int n_runs, int max_run, int heads, int qk_heads,
+                       int dim, int vdim, float q_scale, void* stream);
 /* out[t, h] = o[t, h] / rms(o[t, h]) * w * gate_fn(gate[t, h]) over vdim; gate_kind 0: silu, 1: sigmoid. */
 int qsv_head_rms_gate(void* out, const float* o, const void* w, const void* gate, int64_t gate_stride, int gate_kind, float eps,
                       int n_tokens, int heads, int vdim, int dtype, void* stream);

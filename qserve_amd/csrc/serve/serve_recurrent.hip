@@ -305,6 +305,65 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__
             if (j + c < vdim && r0 + i < dim) Sg[(size_t)(r0 + i) * vdim + j + c] = S[c][i];
 }
 
+// ---- one token per run (decoding): no staging, no barriers - every lane fetches its 8 rows of k, q and the decay itself, the
+// state makes one round trip -----------------------------------------------------------------------------------------------------
+template <typename TQ, typename TB, bool DELTA>
+__global__ __launch_bounds__(256) void recurrent_step_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
+                                                             const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
+                                                             int64_t v_stride, const float* __restrict__ decay,
+                                                             const TB* __restrict__ beta, int64_t beta_stride,
+                                                             float* __restrict__ state, const int32_t* __restrict__ runs, int H,
+                                                             int QH, int dim, int vdim, int lpc_log, float q_scale) {
+    constexpr int R = 8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lpc = 1 << lpc_log, cols = 64 >> lpc_log;
+    const int part = lane & (lpc - 1), j = (blockIdx.z * 4 + wave) * cols + (lane >> lpc_log);
+    const bool col_ok = j < vdim;
+    const int r0 = part * R;
+    const int slot = runs[4 * blockIdx.x];
+    const size_t t = (size_t)runs[4 * blockIdx.x + 1];
+    const bool fresh = runs[4 * blockIdx.x + 3] == 0;
+    const int h = blockIdx.y, qh = h / (H / QH);
+    float* Sg = state + (((size_t)slot * H + h) * dim) * (size_t)vdim + (col_ok ? j : 0);
+    float S[R], kc[R], qc[R], gc[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const bool ok = r0 + i < dim;
+        S[i] = (!fresh && col_ok && ok) ? Sg[(size_t)(r0 + i) * vdim] : 0.f;
+        kc[i] = ok ? ld(k, t * k_stride + (size_t)qh * dim + r0 + i) : 0.f;
+        qc[i] = ok ? ld(q, t * q_stride + (size_t)qh * dim + r0 + i) : 0.f;
+        gc[i] = ok ? decay[(t * H + h) * (size_t)dim + r0 + i] : 0.f;
+    }
+    const float vc = col_ok ? ld(v, t * v_stride + (size_t)h * vdim + j) : 0.f;
+    float acc = 0.f;
+    if (DELTA) {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] *= gc[i];
+            acc += S[i] * kc[i];
+        }
+        const float u = (vc - column_sum(acc, lpc)) / (1.0f + expf(-ld(beta, t * beta_stride + h)));
+        acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] += kc[i] * u;
+            acc += S[i] * qc[i];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] = gc[i] * S[i] + kc[i] * vc;
+            acc += S[i] * qc[i];
+        }
+    }
+    acc = column_sum(acc, lpc);
+    if (!col_ok) return;
+    if (part == 0) o[(t * H + h) * (size_t)vdim + j] = acc * q_scale;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+        if (r0 + i < dim) Sg[(size_t)(r0 + i) * vdim] = S[i];
+}
+
 // ---- per-head RMS norm of the read-out, times a weight shared by the heads, times a gate ---------------------------------------
 // gate_kind 0: silu(g), 1: sigmoid(g)
 template <typename T>
@@ -408,9 +467,32 @@ extern "C" int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, 
 
 extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                                   int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
-                                  int beta_dtype, float* state, const int32_t* runs, int n_runs, int heads, int qk_heads, int dim,
-                                  int vdim, float q_scale, void* stream) {
+                                  int beta_dtype, float* state, const int32_t* runs, int n_runs, int max_run, int heads, int qk_heads,
+                                  int dim, int vdim, float q_scale, void* stream) {
     QSV_REQUIRE(o && q && k && v && decay && state && runs, "qsv_recurrent_scan: null argument");
+    if (max_run == 1 && n_runs > 0 && dim <= 64 * 8 && heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && vdim > 0 && heads <= 65535) {
+        int lpc = 1, lpc_log = 0;
+        while (lpc * 8 < dim) lpc <<= 1, ++lpc_log;
+        const int per_block = 4 * (64 / lpc);
+        const dim3 grid(n_runs, heads, (vdim + per_block - 1) / per_block), block(256);
+        QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
+#define QSV_STEP(TQ, TB, DELTA)                                                                                              \
+    hipLaunchKernelGGL((recurrent_step_kernel<TQ, TB, DELTA>), grid, block, 0, (hipStream_t)stream, o, (const TQ*)q, q_stride,    \
+                       (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state, runs, heads,  \
+                       qk_heads, dim, vdim, lpc_log, q_scale)
+        if (beta) {
+            if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_STEP(float, float, true);
+            else if (qkv_dtype == QSV_F32 && beta_dtype == QSV_BF16) QSV_STEP(float, bf16_t, true);
+            else if (qkv_dtype == QSV_BF16 && beta_dtype == QSV_BF16) QSV_STEP(bf16_t, bf16_t, true);
+            else QSV_REQUIRE(false, "qsv_recurrent_scan: operand types %d / %d", qkv_dtype, beta_dtype);
+        } else {
+            if (qkv_dtype == QSV_F32) QSV_STEP(float, float, false);
+            else if (qkv_dtype == QSV_BF16) QSV_STEP(bf16_t, bf16_t, false);
+            else QSV_REQUIRE(false, "qsv_recurrent_scan: operand type %d", qkv_dtype);
+        }
+#undef QSV_STEP
+        return qsv_launch_status("qsv_recurrent_scan");
+    }
     // Rows of one column per lane: 8 while that leaves the launch at no more than ~2.5 waves per SIMD, else 16 (and for the tallest
     // states).  Measured at 16 heads, 64 x 128 states: 8 x 1024 tokens (2048 / 1024 waves) 0.46 / 0.51 ms plain, 0.50 / 0.55 ms
     // delta rule; 64 single tokens (16384 / 8192 waves) 56 / 43 us; two columns per lane 0.60 / 0.75 ms.  A token's step is a

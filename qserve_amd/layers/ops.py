@@ -261,7 +261,8 @@ class HipOps:
                                              v.stride(0), dtype_code(q.dtype), decay.data_ptr(),
                                              0 if beta is None else beta.data_ptr(), 0 if beta is None else beta.stride(0),
                                              0 if beta is None else dtype_code(beta.dtype), state.data_ptr(), runs.data_ptr(),
-                                             runs.size(0), heads, qk_heads, dim, vdim, float(q_scale), self._s()), "recurrent_scan")
+                                             runs.size(0), max(n for _, _, n in batch.items), heads, qk_heads, dim, vdim,
+                                             float(q_scale), self._s()), "recurrent_scan")
         return o
 
     def head_rms_gate(self, o, w, gate, kind, eps):

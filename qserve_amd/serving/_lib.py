@@ -40,7 +40,7 @@ SIGNATURES = {
     "qsv_glu": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "qsv_decay": (_i, [_vp, _vp, _i64, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
     "qsv_conv_silu_unit": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
-    "qsv_recurrent_scan": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _vp, _i64, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
+    "qsv_recurrent_scan": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _vp, _i64, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
     "qsv_head_rms_gate": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _f, _i, _i, _i, _i, _vp]),
     "qsv_attention_prep": (_i, [_vp, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _f, _vp, _vp, _i, _i, _vp]),
     "qsv_rotate_heads": (_i, [_vp, _vp, _vp, _f, _i, _i, _i, _i, _vp]),

@@ -99,7 +99,7 @@ def test_serve_argument_validation_without_gpu():
     assert L.qsv_latent_attention_mfma_ok(64, 80, 0) == 1 and L.qsv_latent_attention_mfma_ok(64, 80, 1) == 0
     assert L.qsv_latent_attention_mfma_ok(70, 70, 0) == 0
     assert [L.qsv_latent_attention_tile_tokens(h) for h in (1, 3, 6, 16, 32, 40)] == [64, 16, 8, 4, 4, 4]
-    assert L.qsv_recurrent_scan(1, 1, 8, 1, 8, 1, 8, 1, 1, None, 0, 0, 1, 1, 1, 3, 2, 8, 8, 1.0, None) == 1   # 3 heads over 2
+    assert L.qsv_recurrent_scan(1, 1, 8, 1, 8, 1, 8, 1, 1, None, 0, 0, 1, 1, 1, 5, 3, 2, 8, 8, 1.0, None) == 1   # 3 heads over 2
     assert b"heads" in L.qsv_last_error()
     assert L.qsv_hc_write(1, 1, 1, 1, 2, 17, 8, None, None, None, None, 0.0, 0, None) == 1                    # 17 streams
     assert L.qsv_moe_up(1, 1, 1, 1, 1, 1, 8, 7, 2, 0, None) == 1                                              # gated units, odd rows
